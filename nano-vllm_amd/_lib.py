@@ -11,7 +11,8 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip.so")
-ABI_VERSION = 7
+MIXERS_LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip_mixers.so")
+ABI_VERSION = 8
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -60,15 +61,33 @@ PROTOTYPES = {
                                     _i32, _i32, _i32, _i64, _f32, _i64, _i32, _i64, _i64, _i64, _vp]),
 }
 
+# second library (`make mixers`): fp32-stream norms, score-modified attention, recurrent mixers
+MIXERS_PROTOTYPES = {
+    "nv_strerror": (C.c_char_p, [_i32]),
+    "nv_last_error": (C.c_char_p, []),
+    "nv_abi_version": (_i32, []),
+    "nv_add_layernorm": (_i32, [_vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _f32, _vp]),
+    "nv_gelu_tanh_and_mul": (_i32, [_vp, _vp, _i32, _i64, _i32, _i64, _vp]),
+    "nv_qk_prep_store": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _i32, _i32, _i64, _i32, _i32,
+                                _i32, _i32, _i64, _i64, _i64, _vp]),
+    "nv_attn_scoremod_paged": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i32, _i32,
+                                      _i64, _i32, _f32, _f32, _vp, _vp, _i32, _i32, _i64, _i64, _vp]),
+    "nv_causal_conv_silu": (_i32, [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
+    "nv_gated_delta_rule": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
+                                   _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+}
+DTYPE_BF16, DTYPE_F32 = 0, 1
+
 _lock = threading.Lock()
 _lib = None
+_mixers = None
 
 
 class NanoVllmHipError(RuntimeError):
     """A C-ABI call returned a non-zero status."""
 
 
-def load(path: str | None = None) -> C.CDLL:
+def load(path: str | None = None, prototypes: dict | None = None) -> C.CDLL:
     """Load the shared library and attach prototypes.  Raises if it is missing or stale."""
     path = path or os.environ.get("NANOVLLM_HIP_LIB", LIB_PATH)
     if not os.path.exists(path):
@@ -77,7 +96,7 @@ def load(path: str | None = None) -> C.CDLL:
             "`make -C nano-vllm_amd/csrc` (needs hipcc, targets gfx950). There is no CPU fallback."
         )
     dll = C.CDLL(path)
-    for name, (restype, argtypes) in PROTOTYPES.items():
+    for name, (restype, argtypes) in (prototypes if prototypes is not None else PROTOTYPES).items():
         fn = getattr(dll, name)  # AttributeError if the symbol is not exported
         fn.restype = restype
         fn.argtypes = argtypes
@@ -96,9 +115,27 @@ def lib() -> C.CDLL:
     return _lib
 
 
-def check(rc: int, what: str) -> None:
+def mixers() -> C.CDLL:
+    """The second library (libnanovllm_hip_mixers.so)."""
+    global _mixers
+    if _mixers is None:
+        with _lock:
+            if _mixers is None:
+                _mixers = load(os.environ.get("NANOVLLM_HIP_MIXERS_LIB", MIXERS_LIB_PATH), MIXERS_PROTOTYPES)
+    return _mixers
+
+
+def build(target: str = "all") -> None:
+    """Compile the in-tree libraries (`all`), or only the second one (`mixers`), with hipcc for gfx950."""
+    import subprocess
+    jobs = str(min(16, os.cpu_count() or 4))
+    subprocess.run(["make", "-C", os.path.join(_HERE, "csrc"), "-j", jobs, target], check=True,
+                   stdout=subprocess.DEVNULL)
+
+
+def check(rc: int, what: str, dll: C.CDLL | None = None) -> None:
     if rc != 0:
-        dll = lib()
+        dll = dll if dll is not None else lib()
         raise NanoVllmHipError(
             f"{what}: {dll.nv_strerror(rc).decode()} ({rc}): {dll.nv_last_error().decode()}"
         )

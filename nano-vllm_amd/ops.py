@@ -352,3 +352,211 @@ def qknorm_rope_store(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor,
         q.stride(0), k.stride(0), v.stride(0) if store else 0, _stream(q))
     _lib.check(rc, "nv_qknorm_rope_store")
     return q_out, k_out
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Second library: fp32 residual stream + LayerNorm, tanh-GELU gate, score-modified paged attention with free
+# head sizes, short convolution and gated delta rule with per-sequence state slots.  Activations and caches
+# are bfloat16 or float32 (all tensors of one call the same), small per-head / per-channel constants float32.
+# ---------------------------------------------------------------------------------------------------------
+def _dt(t: torch.Tensor, name: str) -> int:
+    _need(t.is_cuda, f"{name} must be a GPU tensor (this path has no CPU implementation)")
+    if t.dtype == _BF16:
+        return _lib.DTYPE_BF16
+    _need(t.dtype == torch.float32, f"{name} must be bfloat16 or float32, got {t.dtype}")
+    return _lib.DTYPE_F32
+
+
+def _f32c(t: Optional[torch.Tensor], name: str) -> int:
+    if t is None:
+        return 0
+    _need(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), f"{name} must be a contiguous float32 GPU tensor")
+    return t.data_ptr()
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _rows2d(t: torch.Tensor, name: str) -> torch.Tensor:
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be [rows, cols] with contiguous columns")
+    return t
+
+
+def add_layernorm(resid: torch.Tensor, h: Optional[torch.Tensor] = None, post: Optional[tuple] = None,
+                  extra: Optional[torch.Tensor] = None, pre: Optional[tuple] = None,
+                  out_dtype: Optional[torch.dtype] = None, eps: float = 1e-5) -> Optional[torch.Tensor]:
+    """One sublayer boundary of an fp32 residual stream, in place on `resid` [T, W]:
+    resid += LN(h; *post) + extra (each part optional); returns y = LN(resid; *pre) in `out_dtype`, or None
+    without `pre`.  post / pre are (weight, bias) float32 [W]."""
+    _need(resid.is_cuda and resid.dtype == torch.float32 and resid.dim() == 2 and resid.is_contiguous(),
+          "resid must be a contiguous float32 [tokens, width] GPU tensor")
+    rows, cols = resid.shape
+    h_dt, h_stride = _lib.DTYPE_F32, cols
+    if h is not None:
+        _rows2d(h, "h")
+        _need(h.shape == resid.shape and post is not None, "h must match resid and come with its (weight, bias)")
+        h_dt, h_stride = _dt(h, "h"), h.stride(0)
+    if extra is not None:
+        _need(extra.shape == resid.shape, "extra must match resid")
+    y, y_dt = None, _lib.DTYPE_F32
+    if pre is not None:
+        y = torch.empty((rows, cols), dtype=out_dtype or torch.float32, device=resid.device)
+        y_dt = _dt(y, "y")
+    for pair, n in ((post, "post"), (pre, "pre")):
+        if pair is not None:
+            _need(pair[0].numel() == cols and pair[1].numel() == cols, f"{n} weight / bias must be [width]")
+    dll = _lib.mixers()
+    rc = dll.nv_add_layernorm(resid.data_ptr(), _ptr(h), h_dt, h_stride,
+                              _f32c(post[0], "post weight") if post and h is not None else None,
+                              _f32c(post[1], "post bias") if post and h is not None else None,
+                              _f32c(extra, "extra") or None,
+                              _f32c(pre[0], "pre weight") if pre else None, _f32c(pre[1], "pre bias") if pre else None,
+                              _ptr(y), y_dt, rows, cols, float(eps), _stream(resid))
+    _lib.check(rc, "nv_add_layernorm", dll)
+    return y
+
+
+def gelu_tanh_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """y = gelu_tanh(gate) * up for x = [gate | up] along the last dimension (fp32 arithmetic, one rounding)."""
+    _rows2d(x, "x")
+    dt = _dt(x, "x")
+    inter = x.shape[1] // 2
+    y = torch.empty((x.shape[0], inter), dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_gelu_tanh_and_mul(x.data_ptr(), y.data_ptr(), dt, x.shape[0], inter, x.stride(0), _stream(x))
+    _lib.check(rc, "nv_gelu_tanh_and_mul", dll)
+    return y
+
+
+def qk_prep_store(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                  slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                  v_cache: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor] = None, rot_dims: int = 0,
+                  temp_coef: float = 0.0, temp_every: int = 0) -> torch.Tensor:
+    """Interleaved-pair rotary on the first rot_dims dimensions of q and k, optional query temperature, scatter of
+    k / v into the paged cache; returns the prepared q [T, H, D]."""
+    dt = _dt(q, "q")
+    for t, n in ((q, "q"), (k, "k"), (v, "v")):
+        _rows_ok(t, n)
+        _need(t.dtype == q.dtype, "q, k, v must have one dtype")
+    T, H, D = q.shape
+    G, Dv = k.shape[1], v.shape[2]
+    _need(k.shape == (T, G, D) and v.shape[:2] == (T, G), "k / v rows do not match q")
+    _need(positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T,
+          "positions must be a contiguous int64 [tokens] GPU tensor")
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "slot_mapping length != number of tokens")
+        _need(k_cache is not None and v_cache is not None and k_cache.is_contiguous() and v_cache.is_contiguous()
+              and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[2:] == (G, D)
+              and v_cache.shape[2:] == (G, Dv) and k_cache.shape[:2] == v_cache.shape[:2],
+              "caches must be contiguous [num_blocks, block_size, G, D] and [.., G, Dv] of q's dtype")
+    if rot_dims:
+        _need(inv_freq is not None and inv_freq.numel() == rot_dims // 2, "inv_freq must hold rot_dims / 2 frequencies")
+    q_out = torch.empty((T, H, D), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_qk_prep_store(q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(), _ptr(k_cache), _ptr(v_cache),
+                              positions.data_ptr(), _ptr(slot_mapping), _f32c(inv_freq, "inv_freq") or None,
+                              int(rot_dims), float(temp_coef), int(temp_every), dt, T, H, G, D, Dv, q.stride(0),
+                              k.stride(0), v.stride(0), _stream(q))
+    _lib.check(rc, "nv_qk_prep_store", dll)
+    return q_out
+
+
+def attn_scoremod_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                        cu_seqlens_k: torch.Tensor, block_tables: torch.Tensor, scale: float, softcap: float = 0.0,
+                        sink: Optional[torch.Tensor] = None, dist_bias: Optional[torch.Tensor] = None,
+                        max_seqlen_q: int = 0, max_seqlen_k: int = 0) -> torch.Tensor:
+    """Causal paged attention with soft-capped scores, a per-head distance bias [H, n_dist] (the last column serves
+    every larger distance) and a per-head sink in the softmax denominator; returns [T, H * Dv]."""
+    dt = _dt(q, "q")
+    _rows_ok(q, "q")
+    T, H, D = q.shape
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.is_contiguous() and v_cache.is_contiguous()
+          and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[:3] == v_cache.shape[:3]
+          and k_cache.shape[3] == D, "caches must be contiguous [num_blocks, block_size, G, D | Dv] of q's dtype")
+    nb, bs, G, _ = k_cache.shape
+    Dv = v_cache.shape[3]
+    _i32(cu_seqlens_q, "cu_seqlens_q")
+    _i32(cu_seqlens_k, "cu_seqlens_k")
+    B = cu_seqlens_k.numel() - 1
+    _need(cu_seqlens_q.numel() == B + 1, "cu_seqlens_q / cu_seqlens_k length mismatch")
+    _need(block_tables.is_cuda and block_tables.dtype == torch.int32 and block_tables.dim() == 2
+          and block_tables.is_contiguous() and block_tables.shape[0] == B,
+          "block_tables must be a contiguous [B, max_blocks] int32 GPU tensor")
+    if sink is not None:
+        _need(sink.numel() == H, "sink must be [H]")
+    n_dist = 0
+    if dist_bias is not None:
+        _need(dist_bias.dim() == 2 and dist_bias.shape[0] == H, "dist_bias must be [H, n_dist]")
+        n_dist = dist_bias.shape[1]
+    out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_attn_scoremod_paged(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+                                    cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), block_tables.data_ptr(), B,
+                                    block_tables.shape[1], T, H, G, D, Dv, nb, bs, float(scale), float(softcap or 0.0),
+                                    _f32c(sink, "sink") or None, _f32c(dist_bias, "dist_bias") or None, n_dist, dt,
+                                    q.stride(0), out.stride(0), _stream(q))
+    _lib.check(rc, "nv_attn_scoremod_paged", dll)
+    return out
+
+
+def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, conv_state: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                     cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor) -> torch.Tensor:
+    """silu(causal conv over time) per channel of x [T, C]; weight [C, taps] float32; conv_state
+    [num_slots, taps - 1, C] (x's dtype) carries each sequence's last inputs and is updated."""
+    dt = _dt(x, "x")
+    _rows2d(x, "x")
+    T, Cc = x.shape
+    taps = weight.shape[1]
+    _need(weight.shape[0] == Cc, "weight must be [channels, taps]")
+    _need(conv_state.is_cuda and conv_state.dtype == x.dtype and conv_state.is_contiguous()
+          and conv_state.shape[1:] == (taps - 1, Cc), "conv_state must be contiguous [slots, taps - 1, C] of x's dtype")
+    for t, n in ((cu_seqlens_q, "cu_seqlens_q"), (cu_seqlens_k, "cu_seqlens_k"), (state_slots, "state_slots")):
+        _i32(t, n)
+    B = state_slots.numel()
+    _need(cu_seqlens_q.numel() == B + 1 and cu_seqlens_k.numel() == B + 1, "one state slot per sequence")
+    y = torch.empty((T, Cc), dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_causal_conv_silu(x.data_ptr(), x.stride(0), _f32c(weight, "weight"), conv_state.data_ptr(),
+                                 y.data_ptr(), y.stride(0), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
+                                 state_slots.data_ptr(), B, T, Cc, taps, dt, _stream(x))
+    _lib.check(rc, "nv_causal_conv_silu", dll)
+    return y
+
+
+def gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a_raw: torch.Tensor, b_raw: torch.Tensor,
+                     gate_raw: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor, norm_weight: torch.Tensor,
+                     state: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
+                     state_slots: torch.Tensor, eps: float) -> torch.Tensor:
+    """Gated delta rule with per-channel decay over a step's rows, state [slots, H, D, Dv] float32 updated in
+    place; q, k: [T, G, D]; v: [T, H, Dv]; a_raw: [T, H * D]; b_raw: [T, H]; gate_raw: [T, H * Dv];
+    returns the normalised, gated read-out [T, H * Dv]."""
+    dt = _dt(q, "q")
+    _rows_ok(q, "q")
+    _rows_ok(k, "k")
+    _rows_ok(v, "v")
+    T, G, D = q.shape
+    H, Dv = v.shape[1], v.shape[2]
+    _need(k.shape == q.shape and v.shape[0] == T, "q / k / v rows differ")
+    for t, n, cols in ((a_raw, "a_raw", H * D), (b_raw, "b_raw", H), (gate_raw, "gate_raw", H * Dv)):
+        _rows2d(t, n)
+        _need(t.shape == (T, cols) and t.dtype == q.dtype, f"{n} must be [T, {cols}] of q's dtype")
+    _need(k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must have one dtype")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, Dv),
+          "state must be contiguous float32 [slots, H, D, Dv]")
+    _need(A_log.numel() == H and dt_bias.numel() == H * D and norm_weight.numel() == Dv, "constant shapes")
+    for t, n in ((cu_seqlens_q, "cu_seqlens_q"), (cu_seqlens_k, "cu_seqlens_k"), (state_slots, "state_slots")):
+        _i32(t, n)
+    B = state_slots.numel()
+    _need(cu_seqlens_q.numel() == B + 1 and cu_seqlens_k.numel() == B + 1, "one state slot per sequence")
+    out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_gated_delta_rule(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0),
+                                 a_raw.data_ptr(), a_raw.stride(0), b_raw.data_ptr(), b_raw.stride(0),
+                                 gate_raw.data_ptr(), gate_raw.stride(0), _f32c(A_log, "A_log"),
+                                 _f32c(dt_bias, "dt_bias"), _f32c(norm_weight, "norm_weight"), state.data_ptr(),
+                                 out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
+                                 state_slots.data_ptr(), B, H, G, D, Dv, float(eps), dt, _stream(q))
+    _lib.check(rc, "nv_gated_delta_rule", dll)
+    return out
