@@ -13,6 +13,7 @@ import torch
 
 from .model_runner import ModelRunner
 from .scheduler import Scheduler
+from .cache_spec import SlotStateSpec
 from .sequence import SamplingParams, Sequence
 
 
@@ -51,18 +52,57 @@ class LLMEngine:
                  max_num_batched_tokens: int = 4000, long_prefill_token_threshold: int = 512,
                  gpu_memory_utilization: float = 0.9, device="cuda", eos: int | None = None,
                  max_num_seqs: int | None = None, tokenizer=None, use_graphs: bool = False,
-                 pipelined_decode: bool = False):
+                 pipelined_decode: bool = False, dtype: torch.dtype = torch.bfloat16):
         """pipelined_decode: decode-only steps are enqueued one ahead of the host: step t+1 is scheduled
         and launched (its input tokens are taken on the device) while step t runs, and the values of
         step t are read afterwards.  Tokens are identical to the synchronous loop; a sequence that
         samples EOS costs one surplus row in the step that was already in flight."""
+        stateful = hasattr(model, "cache_specs") and any(isinstance(c, SlotStateSpec) for c in model.cache_specs())
+        if stateful and max_num_seqs is None:
+            max_num_seqs = 64                 # rows of the state tensors: the most requests live at once
         self.runner = ModelRunner(model, cfg, block_size, num_kvcache_blocks, gpu_memory_utilization, device,
-                                  use_graphs=use_graphs)
+                                  dtype=dtype, use_graphs=use_graphs, num_state_slots=max_num_seqs if stateful else None)
         self.scheduler = Scheduler(self.runner.num_kvcache_blocks, block_size, max_num_batched_tokens,
                                    long_prefill_token_threshold, eos if eos is not None else cfg.eos_token_id,
-                                   max_num_seqs)
+                                   max_num_seqs, num_state_slots=max_num_seqs if stateful else None,
+                                   prefix_caching=getattr(model, "prefix_caching", True))
+        self._replayed: dict[str, Sequence] = {}
         self.tokenizer = tokenizer
         self.pipelined_decode = pipelined_decode
+
+    @classmethod
+    def from_pretrained(cls, model_dir: str, dtype: torch.dtype = torch.bfloat16, device="cuda", **engine_kwargs):
+        """Engine for a checkpoint directory (config.json + *.safetensors): the model class comes from the
+        registry by the architecture the config names."""
+        from ..model.registry import build_model
+        model, cfg = build_model(model_dir, dtype=dtype, device=device)
+        return cls(model, cfg, device=device, dtype=dtype, **engine_kwargs)
+
+    def replay_step(self, entries: list[tuple[str, list[int], list[int]]], end: list[str] = ()) -> torch.Tensor:
+        """One step of a recorded schedule.  entries: (request id, its next token ids, places among them whose
+        logits are asked for); a request is admitted at its first entry and may sit out steps.  All entries run as
+        one batch through the scheduler's bookkeeping, the cache and state manager and the model, as a generated
+        step does; nothing is sampled.  `end`: requests that are finished after this step; their blocks and state
+        slot go back.  Returns float32 logits [asked places, vocab] in the order of the entries."""
+        plan, rows = [], []
+        for rid, tokens, want in entries:
+            seq = self._replayed.get(rid)
+            if seq is None:
+                seq = self._replayed[rid] = Sequence(list(tokens), SamplingParams(0.0, 1))
+                self.scheduler.add(seq)
+            else:
+                seq.extend_prompt(tokens)
+            plan.append((seq, len(tokens)))
+            rows.append(list(want))
+        logits = None
+        if plan:
+            seqs = self.scheduler.schedule_exact(plan)
+            logits = self.runner.forward(seqs, rows)
+            self.scheduler.update_from_output(seqs, [None] * len(seqs))
+        done = [self._replayed.pop(rid) for rid in end if rid in self._replayed]
+        if done:
+            self.scheduler.finish(done)
+        return logits
 
     def add_request(self, prompt, sampling_params: SamplingParams | None = None) -> Sequence:
         if isinstance(prompt, str):

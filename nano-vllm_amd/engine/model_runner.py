@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from ..utils.cache_context import CacheContext, set_context
+from .cache_spec import PagedKVSpec, SlotStateSpec
 from .sequence import Sequence
 
 
@@ -43,6 +44,7 @@ def _prepare_decode_inputs(seqs: list[Sequence], block_size: int) -> dict:
     cu_k = np.zeros(B + 1, dtype=np.int32)
     np.cumsum(start + 1, out=cu_k[1:])
     return dict(input_ids=input_ids, positions=positions, slot_mapping=slots.astype(np.int32), cu_seqlens_q=cu_q,
+                state_slots=np.array([s.state_slot for s in seqs], dtype=np.int32),
                 cu_seqlens_k=cu_k, max_seqlen_q=1, max_seqlen_k=int(start.max()) + 1, block_tables=tables,
                 num_decode_seqs=B, num_leading_decode=B, max_seqlen_k_decode=int(start.max()) + 1,
                 max_seqlen_q_rest=0, max_seqlen_k_rest=0, sum_seqlen_k_decode=int(cu_k[-1]))
@@ -87,6 +89,7 @@ def prepare_inputs(seqs: list[Sequence], block_size: int, decode_fast_path: bool
     single = n_q == 1
     lead = len(seqs) if single.all() else int(np.argmin(single))     # leading rows with one query token
     return dict(input_ids=np.concatenate(ids), positions=np.concatenate(pos),
+                state_slots=np.array([s.state_slot for s in seqs], dtype=np.int32),
                 slot_mapping=np.concatenate(slots).astype(np.int32), cu_seqlens_q=cu_q, cu_seqlens_k=cu_k,
                 max_seqlen_q=int(n_q.max()), max_seqlen_k=int(n_k.max()), block_tables=tables,
                 num_decode_seqs=n_decode, num_leading_decode=lead,
@@ -192,10 +195,19 @@ class _DecodeGraph:
 class ModelRunner:
     def __init__(self, model: torch.nn.Module, cfg, block_size: int = 256, num_kvcache_blocks: int | None = None,
                  gpu_memory_utilization: float = 0.9, device: str | torch.device = "cuda",
-                 dtype: torch.dtype = torch.bfloat16, use_graphs: bool = False):
+                 dtype: torch.dtype = torch.bfloat16, use_graphs: bool = False, num_state_slots: int | None = None):
+        """num_state_slots: rows of the per-sequence state tensors of models with recurrent layers (the most
+        requests that can be live at once)."""
         self.model, self.cfg, self.block_size = model, cfg, block_size
         self.device, self.dtype = torch.device(device), dtype
         self.kv_cache: torch.Tensor | None = None
+        self.cache_specs = model.cache_specs() if hasattr(model, "cache_specs") else None
+        self.num_state_slots = num_state_slots
+        self.has_state = self.cache_specs is not None and any(isinstance(c, SlotStateSpec) for c in self.cache_specs)
+        if self.has_state and not num_state_slots:
+            raise ValueError("this model keeps a state per sequence: num_state_slots (max live requests) must be given")
+        if self.cache_specs is not None and use_graphs:
+            raise ValueError("captured decode graphs are built for the uniform-layer models only")
         self.num_kvcache_blocks = self.init_kv_cache(num_kvcache_blocks, gpu_memory_utilization)
         # Decode steps (one token per sequence) can be replayed from captured HIP graphs: the
         # kernels of a step are launch-latency-bound on small models.  No counterpart in the
@@ -222,6 +234,9 @@ class ModelRunner:
     # ---- KV cache -------------------------------------------------------------------------
     def block_bytes(self) -> int:
         c = self.cfg
+        if self.cache_specs is not None:
+            return sum(spec.block_elems(self.block_size) for spec in self.cache_specs
+                       if isinstance(spec, PagedKVSpec)) * self.dtype.itemsize
         return 2 * c.num_hidden_layers * self.block_size * self.local_kv_heads * c.head_dim * self.dtype.itemsize
 
     @property
@@ -230,8 +245,37 @@ class ModelRunner:
         shard = getattr(self.model, "shard", None)
         return shard.local_kv_heads if shard is not None else self.cfg.num_key_value_heads
 
+    def _init_spec_caches(self, num_blocks: int | None, utilization: float) -> int:
+        """Models that describe their caches (`cache_specs()`): one paged K/V pair per attention run, all sharing
+        the block numbering, and the per-sequence state tensors of the recurrent runs with `num_state_slots` rows."""
+        state_bytes = sum(spec.slot_bytes(self.dtype) for spec in self.cache_specs if isinstance(spec, SlotStateSpec))
+        state_bytes *= self.num_state_slots or 0
+        per_block = self.block_bytes()
+        if num_blocks is None:
+            if self.device.type != "cuda":
+                raise ValueError("num_kvcache_blocks must be given when not running on a GPU")
+            free, total = torch.cuda.mem_get_info(self.device)
+            budget = int(total * utilization) - (total - free) - state_bytes
+            num_blocks = budget // per_block if per_block else 1
+        assert num_blocks > 0, "no memory left for the KV cache"
+        caches = []
+        for spec in self.cache_specs:
+            if isinstance(spec, PagedKVSpec):
+                k = torch.zeros(num_blocks, self.block_size, spec.kv_heads, spec.key_dim, dtype=self.dtype, device=self.device)
+                v = torch.zeros(num_blocks, self.block_size, spec.kv_heads, spec.value_dim, dtype=self.dtype, device=self.device)
+                caches.append((k, v))
+            else:
+                caches.append({name: torch.zeros((self.num_state_slots,) + tuple(shape), dtype=dt or self.dtype,
+                                                 device=self.device)
+                               for name, (shape, dt) in spec.tensors.items()})
+        self.caches = caches
+        self.model.bind_caches(caches)
+        return num_blocks
+
     def init_kv_cache(self, num_blocks: int | None, utilization: float) -> int:
         c = self.cfg
+        if self.cache_specs is not None:
+            return self._init_spec_caches(num_blocks, utilization)
         if num_blocks is None:
             if self.device.type != "cuda":
                 raise ValueError("num_kvcache_blocks must be given when not running on a GPU")
@@ -267,7 +311,8 @@ class ModelRunner:
                            block_size=self.block_size, num_decode_seqs=m["num_decode_seqs"],
                            num_leading_decode=m["num_leading_decode"], max_seqlen_k_decode=m["max_seqlen_k_decode"],
                            max_seqlen_q_rest=m["max_seqlen_q_rest"], max_seqlen_k_rest=m["max_seqlen_k_rest"],
-                           decode_chunk_keys=self._decode_chunk(m, m["max_seqlen_k_decode"]))
+                           decode_chunk_keys=self._decode_chunk(m, m["max_seqlen_k_decode"]),
+                           state_slots=self._to_device(m["state_slots"]) if self.has_state else None)
         set_context(ctx)
         return self._to_device(m["input_ids"]), self._to_device(m["positions"]), m
 
@@ -275,7 +320,7 @@ class ModelRunner:
         """Keys per decode work item for this step's decode rows (0 = the launch plan's choice): the runner knows
         every length, the launch plan only `max_k`, so a few long sequences among many short ones are cut finer."""
         nd = m["num_leading_decode"]
-        if self.device.type != "cuda" or not nd or not self.use_length_hints:
+        if self.device.type != "cuda" or not nd or not self.use_length_hints or self.cache_specs is not None:
             return 0
         from .. import ops
         c = self.cfg
@@ -371,6 +416,33 @@ class ModelRunner:
                 back[i] = tokens[row]
             tokens = back
         return tokens
+
+    @torch.inference_mode()
+    def forward(self, seqs: list[Sequence], rows: list[list[int]] | None = None) -> torch.Tensor:
+        """The step's forward pass without sampling: logits of the asked rows.  rows[i] lists places among sequence
+        i's scheduled tokens (None: every sequence's last scheduled token, what sampling reads); the answer has one
+        row per asked place, in the order of `seqs` and of `rows`.  The batch goes to the model in the runner's own
+        row order, as in `run`."""
+        order = self.step_order(seqs)
+        batch = [seqs[i] for i in order] if order is not None else seqs
+        input_ids, positions, m = self.set_step_context(batch)
+        cu_q = m["cu_seqlens_q"]
+        row_of = {s.id: i for i, s in enumerate(batch)}
+        flat = []
+        for i, s in enumerate(seqs):
+            base, n = int(cu_q[row_of[s.id]]), s.num_scheduled_tokens
+            want = rows[i] if rows is not None else [n - 1]
+            if any(not 0 <= r < n for r in want):
+                raise ValueError(f"{s.id}: asked rows {want} outside its {n} scheduled tokens")
+            flat.extend(base + r for r in want)
+        if not flat:
+            flat = [0]                                 # the pass still runs: it fills the cache and the state
+            keep = 0
+        else:
+            keep = len(flat)
+        logits_rows = torch.tensor(flat, dtype=torch.int64).to(self.device)
+        logits = self.model(input_ids, positions, logits_rows=logits_rows)
+        return logits[:keep]
 
     @torch.inference_mode()
     def run(self, seqs: list[Sequence]) -> list[int | None]:

@@ -20,17 +20,24 @@ from collections import deque
 
 from .block_manager import BlockManager
 from .sequence import PENDING, Sequence, SequenceStatus
+from .state_manager import StateSlotManager
 
 
 class Scheduler:
     def __init__(self, num_kvcache_blocks: int, kvcache_block_size: int = 256, max_num_batched_tokens: int = 4000,
-                 long_prefill_token_threshold: int = 512, eos: int | None = None, max_num_seqs: int | None = None):
+                 long_prefill_token_threshold: int = 512, eos: int | None = None, max_num_seqs: int | None = None,
+                 num_state_slots: int | None = None, prefix_caching: bool = True):
+        """num_state_slots: models with recurrent layers keep a state per sequence in numbered slots; a request is
+        admitted only while a slot is free and gives it back when it ends or is preempted.  prefix_caching=False for
+        such models: a cached prefix has no recurrent state to continue from."""
         self.block_size = kvcache_block_size
         self.max_scheduled_tokens = max_num_batched_tokens
         self.long_prefill_token_threshold = long_prefill_token_threshold
         self.eos = eos
         self.max_num_seqs = max_num_seqs
         self.block_manager = BlockManager(num_kvcache_blocks, kvcache_block_size)
+        self.state_slots = StateSlotManager(num_state_slots) if num_state_slots else None
+        self.prefix_caching = prefix_caching
         self.waiting: deque[Sequence] = deque()
         self.running: deque[Sequence] = deque()
 
@@ -80,7 +87,8 @@ class Scheduler:
                         break
             if got:
                 seq.num_scheduled_tokens = n_new
-                bm.publish_full_blocks(seq, seq.num_computed_tokens + n_new)
+                if self.prefix_caching:
+                    bm.publish_full_blocks(seq, seq.num_computed_tokens + n_new)
                 budget -= n_new
                 scheduled.append(seq)
                 i += 1
@@ -95,9 +103,11 @@ class Scheduler:
         while self.waiting and budget > 0 and not preempted:
             if self.max_num_seqs is not None and len(self.running) >= self.max_num_seqs:
                 break
+            if self.state_slots is not None and not self.state_slots.can_allocate():
+                break
             seq = self.waiting[0]
             tokens = seq.token_ids if seq.output_tokens else seq.prompt_tokens   # all of it after a preemption
-            cached_blocks, n_cached = bm.get_computed_blocks(tokens)
+            cached_blocks, n_cached = bm.get_computed_blocks(tokens) if self.prefix_caching else ([], 0)
             n_new = len(tokens) - n_cached
             if 0 < self.long_prefill_token_threshold < n_new:
                 n_new = self.long_prefill_token_threshold
@@ -109,11 +119,14 @@ class Scheduler:
             if not bm.can_allocate(max(blocks_needed, blocks_whole) + idle_hits):
                 break
             bm.allocate_slots(seq, cached_blocks, blocks_needed)
+            if self.state_slots is not None:
+                seq.state_slot = self.state_slots.allocate(seq.id)
             seq.num_computed_tokens = n_cached
             seq.num_cached_tokens = n_cached
             seq.num_scheduled_tokens = n_new
             seq.status = SequenceStatus.RUNNING
-            bm.publish_full_blocks(seq, n_cached + n_new)
+            if self.prefix_caching:
+                bm.publish_full_blocks(seq, n_cached + n_new)
             budget -= n_new
             self.waiting.popleft()
             self.running.append(seq)
@@ -139,15 +152,65 @@ class Scheduler:
     def _preempt(self, seq: Sequence) -> None:
         """Recompute-preemption: release the blocks, forget the computed count, back to waiting."""
         self.block_manager.free_sequence(seq.id)
+        self._release_slot(seq)
         seq.block_table = []
         seq.num_computed_tokens = 0
         seq.num_scheduled_tokens = 0
         seq.num_preemptions += 1
         seq.status = SequenceStatus.WAITING
 
+    def _release_slot(self, seq: Sequence) -> None:
+        if self.state_slots is not None:
+            self.state_slots.free(seq.id)
+            seq.state_slot = -1
+
+    def schedule_exact(self, plan: list[tuple[Sequence, int]]) -> list[Sequence]:
+        """A step that is given, not chosen: each (sequence, n) runs its next n tokens, in this order.  A sequence
+        that is not running yet is admitted (blocks for these tokens, a state slot); a running one grows.  Replays
+        of recorded schedules use it; nothing is preempted: a step that does not fit the cache raises ValueError
+        and leaves the scheduler as it was before the step, apart from blocks already grown."""
+        bm = self.block_manager
+        for seq, n in plan:
+            if n < 1 or seq.num_computed_tokens + n > len(seq):
+                raise ValueError(f"{seq.id}: cannot run {n} tokens from {seq.num_computed_tokens} of {len(seq)}")
+        scheduled = []
+        for seq, n in plan:
+            if seq.status == SequenceStatus.WAITING:
+                if self.state_slots is not None and not self.state_slots.can_allocate():
+                    raise ValueError("no free state slot")
+                blocks = -(-n // self.block_size)
+                if not bm.can_allocate(blocks):
+                    raise ValueError(f"{seq.id}: the cache cannot hold {n} tokens")
+                bm.allocate_slots(seq, [], blocks)
+                if self.state_slots is not None:
+                    seq.state_slot = self.state_slots.allocate(seq.id)
+                seq.num_computed_tokens = seq.num_cached_tokens = 0
+                seq.status = SequenceStatus.RUNNING
+                self.waiting.remove(seq)
+                self.running.append(seq)
+            else:
+                bm.append_slots(seq, n)
+            seq.num_scheduled_tokens = n
+            if self.prefix_caching:
+                bm.publish_full_blocks(seq, seq.num_computed_tokens + n)
+            scheduled.append(seq)
+        for seq in self.running:
+            if seq not in scheduled:
+                seq.num_scheduled_tokens = 0
+        return scheduled
+
+    def finish(self, seqs: list[Sequence]) -> None:
+        """End requests from outside (a replay's own end marks): blocks and state slots go back."""
+        for seq in seqs:
+            seq.status = SequenceStatus.FINISHED
+            if seq in self.waiting:
+                self.waiting.remove(seq)
+        self._retire(seqs)
+
     def _retire(self, finished: list[Sequence]) -> None:
         for seq in finished:
             self.block_manager.free_sequence(seq.id)
+            self._release_slot(seq)
             seq.block_table = []
         self.running = deque(s for s in self.running if not s.is_finished)
 

@@ -40,6 +40,7 @@ class Sequence:
         self.num_pending = 0              # trailing output tokens that are still PENDING (0 or 1)
         self.stopped_early = False        # finished on EOS while a later step was already in flight
         self.num_preemptions = 0          # times its blocks were taken away and its K/V recomputed
+        self.state_slot = -1              # row of the per-sequence state tensors (models with recurrent layers)
         self.sampling_params = sampling_params or SamplingParams()
 
     def __len__(self) -> int:
@@ -74,6 +75,13 @@ class Sequence:
     def token_at(self, pos: int) -> int:
         n = len(self.prompt_tokens)
         return self.prompt_tokens[pos] if pos < n else self.output_tokens[pos - n]
+
+    def extend_prompt(self, token_ids: list[int]) -> None:
+        """More given tokens for a request that is fed piece by piece (replaying a recorded schedule): they count
+        as prompt, and only before anything was sampled."""
+        if self.output_tokens:
+            raise ValueError("cannot extend the prompt of a sequence that has sampled tokens")
+        self.prompt_tokens.extend(token_ids)
 
     def add_token(self, token_id: int) -> None:
         self.output_tokens.append(token_id)

@@ -14,3 +14,10 @@ class SiluAndMul(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.silu_and_mul(x)
+
+
+class GeluTanhAndMul(nn.Module):
+    """gelu_tanh(gate) * up for x = [gate | up] (the HIP kernel ``nv_gelu_tanh_and_mul``; bfloat16 or float32)."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.gelu_tanh_and_mul(x)

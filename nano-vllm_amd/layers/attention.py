@@ -119,3 +119,46 @@ class Attention(nn.Module):
                 "through the paged cache (bind per-layer views before the first forward)")
         self.store_kvcache(k, v, ctx.slot_mapping, ctx.block_size)
         return self.attend(q)
+
+
+class ScoreModAttention(nn.Module):
+    """Causal paged attention for designs the fixed kernels above do not cover: key size and value size are free
+    and may differ, scores are fp32 and may be soft-capped (cap * tanh(s / cap)), a per-head learned sink may sit in
+    the softmax denominator, a per-head distance bias may be added to the capped score, q and k may get a partial
+    interleaved-pair rotary, and q a position-dependent temperature.  bfloat16 or float32 operands.
+
+    The module owns no cache: a layer that runs several times per forward (weight-shared passes) has one cache
+    per run, so the caches are arguments: k_cache [num_blocks, block_size, G, D], v_cache [.., G, Dv].
+    """
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int, scale: float,
+                 softcap: float = 0.0, rot_dims: int = 0, rot_base: float = 10000.0, temp_coef: float = 0.0,
+                 temp_every: int = 0, use_sink: bool = False, device=None):
+        super().__init__()
+        assert num_heads % num_kv_heads == 0
+        self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim = num_heads, num_kv_heads, head_dim, v_head_dim
+        self.scale, self.softcap = float(scale), float(softcap or 0.0)
+        self.rot_dims, self.temp_coef, self.temp_every = int(rot_dims), float(temp_coef), int(temp_every)
+        if self.rot_dims:
+            # base^(-2i/dims) in double precision, rounded once; the angle is the fp32 product position * frequency
+            i = torch.arange(self.rot_dims // 2, dtype=torch.float64)
+            inv = (float(rot_base) ** (-2.0 * i / self.rot_dims)).to(torch.float32)
+            self.register_buffer("inv_freq", inv.to(device) if device is not None else inv, persistent=False)
+        else:
+            self.inv_freq = None
+        self.sink = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32, device=device)) if use_sink else None
+        self.dist_bias: torch.Tensor | None = None     # [H, n_dist] float32, set by the owner (set_distance_bias)
+
+    def set_distance_bias(self, table: torch.Tensor | None) -> None:
+        """table[h, n] is added to the score of a key n positions back; the last column serves all larger n."""
+        self.dist_bias = None if table is None else table.to(torch.float32).contiguous()
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor,
+                k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+        """q [T, H, D], k [T, G, D], v [T, G, Dv] as projected; returns [T, H * Dv]."""
+        ctx = get_context()
+        q = ops.qk_prep_store(positions, q, k, v, ctx.slot_mapping, k_cache, v_cache, self.inv_freq, self.rot_dims,
+                              self.temp_coef, self.temp_every)
+        return ops.attn_scoremod_paged(q, k_cache, v_cache, ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.block_tables,
+                                       self.scale, self.softcap, self.sink, self.dist_bias, ctx.max_seqlen_q,
+                                       ctx.max_seqlen_k)

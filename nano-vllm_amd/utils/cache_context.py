@@ -50,6 +50,9 @@ class CacheContext:
     # (`ops.decode_suggest_chunk`: a few long sequences among many short ones); 0 = the launch plan decides
     # from `max_seqlen_k` alone.
     decode_chunk_keys: int = 0
+    # Extension (optional): [B] int32, the state slot of every sequence of the step, for layers that carry a
+    # recurrent state per sequence (layers/delta_rule.py).  None for models without such layers.
+    state_slots: Optional[torch.Tensor] = None
 
 
 _cache_context: ContextVar[Optional[CacheContext]] = ContextVar("CacheContext", default=None)

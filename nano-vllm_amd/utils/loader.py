@@ -17,6 +17,16 @@ def load_model(model: torch.nn.Module, model_path: str, strict: bool = True) -> 
     files = sorted(glob.glob(os.path.join(model_path, "*.safetensors")))
     if not files:
         raise FileNotFoundError(f"no *.safetensors under {model_path}")
+    if hasattr(model, "load_tensors"):
+        # a model whose checkpoint names are not its parameter names (or whose files fix some of its sizes) places
+        # the tensors itself
+        tensors = {}
+        for path in files:
+            with safe_open(path, framework="pt", device="cpu") as f:
+                for name in f.keys():
+                    tensors[name] = f.get_tensor(name)
+        model.load_tensors(tensors)
+        return []
     shard = getattr(model, "shard", None)
     d = model.config.head_dim if shard is not None else 0
     params = dict(model.named_parameters())
