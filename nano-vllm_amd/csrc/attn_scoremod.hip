@@ -18,6 +18,7 @@
 // query temperature q *= 1 + coef * ln(floor((p + 1) / every) + 1), and the scatter of the step's K/V rows into the
 // cache.
 #include "nv_common.h"
+#include "../../include/nanovllm_hip_mixers.h"
 
 namespace nv {
 

@@ -23,6 +23,7 @@
 #include <algorithm>
 
 #include "nv_common.h"
+#include "../../include/nanovllm_hip_mixers.h"
 
 namespace nv {
 

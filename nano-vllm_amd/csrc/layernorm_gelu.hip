@@ -12,6 +12,7 @@
 // passes over a row held in registers (mean first, then squared deviations), eps inside the root.
 // One workgroup of 256 threads per row; a thread holds up to kMaxPerThread elements.
 #include "nv_common.h"
+#include "../../include/nanovllm_hip_mixers.h"
 
 namespace nv {
 

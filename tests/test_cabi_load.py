@@ -13,9 +13,25 @@ import nanovllm_amd
 from nanovllm_amd import _lib, ops
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "nanovllm_hip.h")).read()
+def declared_symbols(header="nanovllm_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     return re.findall(r"NV_API\s+[\w\s\*]+?\b(nv_\w+)\s*\(", text)
+
+
+def test_second_library_header_prototypes_and_exports_agree():
+    syms = declared_symbols("nanovllm_hip_mixers.h")
+    common = {"nv_strerror", "nv_last_error", "nv_abi_version"}
+    assert len(syms) == len(set(syms)) and set(syms) | common == set(_lib.MIXERS_PROTOTYPES)
+    dll = _lib.mixers()
+    for name in syms:
+        assert hasattr(dll, name), f"{name} not exported"
+    assert dll.nv_abi_version() == _lib.ABI_VERSION
+    # argument errors are reported before any device access
+    assert dll.nv_add_layernorm(None, None, 0, 0, None, None, None, None, None, None, 0, 4, 64, 1e-5, None) == -1
+    assert b"null residual" in dll.nv_last_error()
+    assert dll.nv_causal_conv_silu(None, 0, None, None, None, 0, None, None, None, 1, 4, 8, 9, 0, None) == -2
+    assert dll.nv_gated_delta_rule(None, None, None, 0, 0, 0, None, 0, None, 0, None, 0, None, None, None, None, None,
+                                   0, None, None, None, 0, 2, 2, 8, 8, 1e-5, 0, None) == 0       # no sequences: a no-op
 
 
 def test_header_declares_expected_entry_points():
