@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ cu_k, const int* __restrict__ block_tables, int B,
     int max_blocks, int H, int G, int D, int Dv, int block_size, float scale, float softcap,
     const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride) {
+    int64_t out_stride, int only_single_rows) {
     extern __shared__ float smem[];
     float* qs = smem;                      // [D]
     float* ps = smem + D;                  // [64]
@@ -102,6 +102,7 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
     }
     const int b = lo;
     const int len_q = cu_q[b + 1] - cu_q[b], len_k = cu_k[b + 1] - cu_k[b];
+    if (only_single_rows && len_q != 1) return;          // the tile kernel has the sequences with several rows
     const int pos = len_k - len_q + (t - cu_q[b]);      // this query's position; it sees keys 0 .. pos
     const int g = h / (H / G);
     for (int d = lane; d < D; d += 64) qs[d] = (float)q[(int64_t)t * q_stride + (int64_t)h * D + d];
@@ -166,6 +167,167 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------ prompt portions
+// bf16 MFMA kernel for sequences with several query rows.  A workgroup of four waves takes 64 consecutive queries of
+// one (sequence, head); a wave owns 16 of them.  Key tiles of 64 go through LDS once per workgroup: K as stored
+// ([key][d]) and V transposed ([dv][key]).  Everything is computed transposed, so that one lane keeps one query:
+//     S^T (keys x queries) = K Q^T        v_mfma_f32_16x16x16_bf16: A = K rows from LDS, B = Q^T held in registers
+//     O^T (dv x queries)  += V^T P^T      A = V^T rows from LDS, B = P^T, which is the accumulator layout of S^T as is
+// Lane l holds query l % 16 in every accumulator, so the running maximum, the rescale factor and the denominator are
+// per-lane scalars (the maximum joins the four lane groups with two shuffles per tile, the denominator once at the end).
+constexpr int kTileQ = 64, kTileK = 64, kTileThreads = 256;
+
+__device__ __forceinline__ float fast_tanh(float x) {
+    // 1 - 2 / (e^{2x} + 1): exact limits at both ends (e^{2x} -> inf gives 1, -> 0 gives -1)
+    return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f);
+}
+
+template <int NS>     // NS: most 16-wide steps over D and over Dv (D, Dv <= 16 * NS)
+__global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+    __bf16* __restrict__ out, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
+    const int* __restrict__ block_tables, int max_blocks, int tiles_per_seq, int H, int G, int D, int Dv,
+    int block_size, float scale, float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias,
+    int n_dist, int64_t q_stride, int64_t out_stride) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int b = blockIdx.x / tiles_per_seq, qt = blockIdx.x % tiles_per_seq, h = blockIdx.y;
+    const int q0 = cu_q[b], len_q = cu_q[b + 1] - q0, len_k = cu_k[b + 1] - cu_k[b];
+    if (len_q <= 1 || qt * kTileQ >= len_q) return;          // single rows belong to the row-wave kernel
+    const int g = h / (H / G);
+    const int ds = D / 16, dvs = Dv / 16;
+    const int k_ld = D + 8, v_ld = kTileK + 8;                // LDS row lengths in elements (16-byte multiples)
+    __bf16* ldsK = (__bf16*)lds_raw;                          // [64][D + 8]
+    __bf16* ldsV = ldsK + kTileK * k_ld;                      // [Dv][64 + 8]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 15, lg = lane >> 4;
+    const int start = len_k - len_q;                          // position of the sequence's first row in this step
+    const int row0 = qt * kTileQ + wave * 16;                 // first query of this wave (index within the step's rows)
+    const int my_row = min(row0 + lq, len_q - 1);             // rows past the end repeat the last one and are not stored
+    const int my_pos = start + my_row;
+    const int wave_last_pos = start + min(row0 + 15, len_q - 1);
+    const bool wave_live = row0 < len_q;
+    // Q^T fragments: lane holds q[my_row][16 s + 4 lg .. + 3]
+    s16x4 qf[NS];
+    {
+        const __bf16* qr = q + (int64_t)(q0 + my_row) * q_stride + (int64_t)h * D;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            qf[s] = s < ds ? *(const s16x4*)(qr + 16 * s + 4 * lg) : s16x4{0, 0, 0, 0};
+    }
+    f32x4 oacc[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const int* table = block_tables + (int64_t)b * max_blocks;
+    const float* bias_h = dist_bias ? dist_bias + (int64_t)h * n_dist : nullptr;
+    const int last_pos = start + min(qt * kTileQ + kTileQ, len_q) - 1;      // the tile's last query sees keys 0 .. last_pos
+    const int kchunks = D / 8, vchunks = Dv / 8;
+    for (int base = 0; base <= last_pos; base += kTileK) {
+        __syncthreads();                                      // the previous tile has been consumed
+        for (int c = tid; c < kTileK * kchunks; c += kTileThreads) {
+            const int key = c / kchunks, ch = c - key * kchunks, j = base + key;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (j < len_k) {
+                const int64_t row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
+                val = *(const uint4*)(k_cache + row * D + 8 * ch);
+            }
+            *(uint4*)(ldsK + key * k_ld + 8 * ch) = val;
+        }
+        for (int c = tid; c < kTileK * vchunks; c += kTileThreads) {
+            const int key = c / vchunks, ch = c - key * vchunks, j = base + key;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (j < len_k) {
+                const int64_t row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
+                val = *(const uint4*)(v_cache + row * Dv + 8 * ch);
+            }
+            const unsigned short* e = (const unsigned short*)&val;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ((unsigned short*)ldsV)[(8 * ch + i) * v_ld + key] = e[i];
+        }
+        __syncthreads();
+        if (!wave_live || base > wave_last_pos) continue;     // (uniform per wave; the barriers above stay matched)
+        // ---- S^T for four 16-key blocks -----------------------------------------------------------------------
+        f32x4 sacc[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            sacc[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                if (s < ds) {
+                    const s16x4 a = *(const s16x4*)(ldsK + (kb * 16 + lq) * k_ld + 16 * s + 4 * lg);
+                    sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sacc[kb], 0, 0, 0);
+                }
+            }
+        }
+        // ---- modifiers, mask, running maximum -----------------------------------------------------------------
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = base + kb * 16 + 4 * lg + i;
+                float sc = sacc[kb][i] * scale;
+                if (softcap > 0.f) sc = softcap * fast_tanh(sc / softcap);
+                if (bias_h) sc += bias_h[min(max(my_pos - j, 0), n_dist - 1)];
+                sc = j <= my_pos ? sc : -INFINITY;
+                sacc[kb][i] = sc;
+                tmax = fmaxf(tmax, sc);
+            }
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float m_new = fmaxf(m, tmax);                   // finite from the first tile on: key 0 is visible to all
+        const float corr = __expf(m - m_new);
+        m = m_new;
+        l *= corr;
+#pragma unroll
+        for (int i = 0; i < NS; ++i) oacc[i] *= corr;
+        // ---- P^T, then O^T += V^T P^T ---------------------------------------------------------------------------
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            float p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[i] = __expf(sacc[kb][i] - m_new);
+                l += p[i];
+            }
+            const uint32_t p01 = pack_bf16(p[0], p[1]), p23 = pack_bf16(p[2], p[3]);
+            const s16x4 pb = __builtin_bit_cast(s16x4, make_uint2(p01, p23));
+#pragma unroll
+            for (int dv = 0; dv < NS; ++dv) {
+                if (dv < dvs) {
+                    const s16x4 a = *(const s16x4*)(ldsV + (dv * 16 + lq) * v_ld + kb * 16 + 4 * lg);
+                    oacc[dv] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dv], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!wave_live) return;
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    if (sink) {
+        const float sk = sink[h];
+        const float m_new = fmaxf(m, sk);
+        const float corr = __expf(m - m_new);
+        l = l * corr + __expf(sk - m_new);
+#pragma unroll
+        for (int i = 0; i < NS; ++i) oacc[i] *= corr;
+    }
+    if (row0 + lq < len_q) {
+        const float inv = 1.0f / l;
+        __bf16* orow = out + (int64_t)(q0 + row0 + lq) * out_stride + (int64_t)h * Dv;
+#pragma unroll
+        for (int dv = 0; dv < NS; ++dv) {
+            if (dv < dvs) {
+                const uint2 pk = make_uint2(pack_bf16(oacc[dv][0] * inv, oacc[dv][1] * inv),
+                                            pack_bf16(oacc[dv][2] * inv, oacc[dv][3] * inv));
+                *(uint2*)(orow + dv * 16 + 4 * lg) = pk;
+            }
+        }
+    }
+}
+
 }  // namespace nv
 
 extern "C" int nv_qk_prep_store(const void* q, const void* k, const void* v, void* q_out, void* k_cache,
@@ -201,8 +363,8 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
                                       const int* cu_seqlens_q, const int* cu_seqlens_k, const int* block_tables,
                                       int num_seqs, int max_blocks_per_seq, int64_t T, int H, int G, int D, int Dv,
                                       int64_t num_blocks, int block_size, float scale, float softcap,
-                                      const float* sink, const float* dist_bias, int n_dist, int dtype,
-                                      int64_t q_stride, int64_t out_stride, void* stream) {
+                                      const float* sink, const float* dist_bias, int n_dist, int max_seqlen_q,
+                                      int single_rows, int dtype, int64_t q_stride, int64_t out_stride, void* stream) {
     using namespace nv;
     NV_REQUIRE(num_seqs >= 0 && T >= 0 && H > 0 && G > 0 && D > 0 && Dv > 0 && block_size > 0 && num_blocks > 0 &&
                    max_blocks_per_seq > 0,
@@ -218,17 +380,42 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_attn_scoremod_paged: bad dtype");
     NV_REQUIRE(T < (1LL << 31) && H < 65536, NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: launch too large");
     hipStream_t s = (hipStream_t)stream;
+    // Sequences with several rows go to the MFMA tile kernel when the shapes allow (bf16, head sizes in multiples of
+    // 16 up to 256, tiles within 64 KiB of LDS, 16-byte aligned rows); the row-wave kernel then takes the single rows
+    // only.  max_seqlen_q <= 0 (unknown) or 1 keeps everything on the row-wave kernel.
+    int only_single = 0;
+    const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 8) + (size_t)Dv * (kTileK + 8));
+    if (dtype == NV_DTYPE_BF16 && max_seqlen_q > 1 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 &&
+        tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
+        ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0) {
+        const int tiles = (max_seqlen_q + kTileQ - 1) / kTileQ;
+        NV_REQUIRE((int64_t)num_seqs * tiles < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: launch too large");
+        const dim3 tgrid((unsigned)(num_seqs * tiles), (unsigned)H);
+#define NV_TILE_ARGS                                                                                                  \
+    (const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q, cu_seqlens_k,      \
+        block_tables, max_blocks_per_seq, tiles, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,  \
+        q_stride, out_stride
+        if (D <= 128 && Dv <= 128)
+            hipLaunchKernelGGL(attn_scoremod_tile_kernel<8>, tgrid, dim3(kTileThreads), tile_lds, s, NV_TILE_ARGS);
+        else
+            hipLaunchKernelGGL(attn_scoremod_tile_kernel<16>, tgrid, dim3(kTileThreads), tile_lds, s, NV_TILE_ARGS);
+#undef NV_TILE_ARGS
+        const int rc = check_launch("nv_attn_scoremod_paged (tile kernel)");
+        if (rc != NV_OK) return rc;
+        if (single_rows == 0) return NV_OK;
+        only_single = 1;
+    }
     const size_t smem = sizeof(float) * (D + 64 + (D & 1)) + sizeof(int64_t) * 64;
     const dim3 grid((unsigned)T, (unsigned)H);
     if (dtype == NV_DTYPE_BF16)
         hipLaunchKernelGGL(attn_scoremod_rowwave_kernel<__bf16>, grid, dim3(64), smem, s, (const __bf16*)q,
                            (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q, cu_seqlens_k,
                            block_tables, num_seqs, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink,
-                           dist_bias, n_dist, q_stride, out_stride);
+                           dist_bias, n_dist, q_stride, out_stride, only_single);
     else
         hipLaunchKernelGGL(attn_scoremod_rowwave_kernel<float>, grid, dim3(64), smem, s, (const float*)q,
                            (const float*)k_cache, (const float*)v_cache, (float*)out, cu_seqlens_q, cu_seqlens_k,
                            block_tables, num_seqs, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink,
-                           dist_bias, n_dist, q_stride, out_stride);
+                           dist_bias, n_dist, q_stride, out_stride, only_single);
     return check_launch("nv_attn_scoremod_paged");
 }

@@ -159,6 +159,7 @@ class ScoreModAttention(nn.Module):
         ctx = get_context()
         q = ops.qk_prep_store(positions, q, k, v, ctx.slot_mapping, k_cache, v_cache, self.inv_freq, self.rot_dims,
                               self.temp_coef, self.temp_every)
+        singles = -1 if ctx.num_decode_seqs is None else int(ctx.num_decode_seqs > 0)
         return ops.attn_scoremod_paged(q, k_cache, v_cache, ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.block_tables,
                                        self.scale, self.softcap, self.sink, self.dist_bias, ctx.max_seqlen_q,
-                                       ctx.max_seqlen_k)
+                                       ctx.max_seqlen_k, singles)

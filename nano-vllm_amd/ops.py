@@ -466,7 +466,7 @@ def qk_prep_store(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: 
 def attn_scoremod_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cu_seqlens_q: torch.Tensor,
                         cu_seqlens_k: torch.Tensor, block_tables: torch.Tensor, scale: float, softcap: float = 0.0,
                         sink: Optional[torch.Tensor] = None, dist_bias: Optional[torch.Tensor] = None,
-                        max_seqlen_q: int = 0, max_seqlen_k: int = 0) -> torch.Tensor:
+                        max_seqlen_q: int = 0, max_seqlen_k: int = 0, single_rows: int = -1) -> torch.Tensor:
     """Causal paged attention with soft-capped scores, a per-head distance bias [H, n_dist] (the last column serves
     every larger distance) and a per-head sink in the softmax denominator; returns [T, H * Dv]."""
     dt = _dt(q, "q")
@@ -495,8 +495,8 @@ def attn_scoremod_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     rc = dll.nv_attn_scoremod_paged(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
                                     cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), block_tables.data_ptr(), B,
                                     block_tables.shape[1], T, H, G, D, Dv, nb, bs, float(scale), float(softcap or 0.0),
-                                    _f32c(sink, "sink") or None, _f32c(dist_bias, "dist_bias") or None, n_dist, dt,
-                                    q.stride(0), out.stride(0), _stream(q))
+                                    _f32c(sink, "sink") or None, _f32c(dist_bias, "dist_bias") or None, n_dist,
+                                    int(max_seqlen_q), int(single_rows), dt, q.stride(0), out.stride(0), _stream(q))
     _lib.check(rc, "nv_attn_scoremod_paged", dll)
     return out
 

@@ -128,6 +128,36 @@ def test_scoremod_attention_mixed_batch(dtype, shape, flavour):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 2, 96, 96), (2, 2, 128, 64), (4, 1, 32, 160), (2, 1, 256, 256)])
+def test_scoremod_attention_long_portions_cross_query_and_key_tiles(dtype, shape):
+    """Portions longer than the MFMA kernel's 64-query tile over caches longer than its 64-key tile, pages of 24
+    (no multiple of either), single rows in between, and a sequence of 65 rows (one row into the second tile)."""
+    H, G, D, Dv = shape
+    bs, nb = 24, 60
+    n_qs, n_ks = [200, 1, 130, 65, 2], [200, 77, 300, 65, 130]
+    a, r = _attention_pair(H, G, D, Dv, scale=D ** -0.5, softcap=25.0, rot_dims=16, rot_base=1000.0, use_sink=True)
+    g = torch.Generator(device=DEV).manual_seed(7)
+    table = torch.randn(H, 90, generator=g, device=DEV)
+    a.set_distance_bias(table)
+    r.set_distance_bias(table)
+    with torch.no_grad():
+        a.sink.copy_(torch.randn(H, generator=g, device=DEV))
+        r.sink.copy_(a.sink)
+    ctx, pos = _context(n_qs, n_ks, bs, nb, seed=4)
+    ctx.num_decode_seqs = 1
+    T = sum(n_qs)
+    mk = lambda *s: torch.randn(*s, generator=g, device=DEV).to(dtype)
+    kc, vc = mk(nb, bs, G, D), mk(nb, bs, G, Dv)
+    kc_r, vc_r = kc.clone(), vc.clone()
+    q, k, v = mk(T, H, D), mk(T, G, D), mk(T, G, Dv)
+    nv.set_context(ctx)
+    o = a(q, k, v, pos, kc, vc)
+    o_r = r(q, k, v, pos, kc_r, vc_r)
+    nv.set_context(None)
+    torch.testing.assert_close(o.float(), o_r.float(), **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 3, 4])
 def test_short_conv_in_portions_matches_one_pass(dtype, taps):
     C, slots_n = 200, 5
