@@ -62,6 +62,9 @@ def parse():
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end generation run (N=1 only)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-attention records (rank 0)")
     ap.add_argument("--no-configs", action="store_true", help="skip the decode records at config 4 / 5 shapes (rank 0)")
+    ap.add_argument("--buvalix", action="store_true",
+                    help="instead of the default workload: the Buvalix kernels and model beside the Qwen3 path at "
+                         "equal sizes (one GPU, random weights), one JSON line")
     return ap.parse_args()
 
 
@@ -782,6 +785,12 @@ def dp_config5_bench(args, dev, rank, world, dist):
 
 def main():
     args = parse()
+    if args.buvalix:
+        if not torch.cuda.is_available():
+            raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
+        from tools.buvalix_bench import run as buvalix_run
+        print(json.dumps(buvalix_run("cuda:0")))
+        return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))

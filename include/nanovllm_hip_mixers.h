@@ -61,18 +61,21 @@ NV_API int nv_qk_prep_store(const void* q, const void* k, const void* v, void* q
  * q: [T, H, D] (token stride q_stride), out: [T, H, Dv] (token stride out_stride);
  * k_cache: [num_blocks, block_size, G, D], v_cache: [num_blocks, block_size, G, Dv]; query i of sequence b sits at
  * position len_k(b) - len_q(b) + i.  Dv <= 256.
- * max_seqlen_q: the most rows any sequence has in this step (0 = unknown).  With bf16 and head sizes in multiples of
- * 16, sequences with several rows run on an MFMA tile kernel sized from it and single rows on the row-per-wave
- * kernel; single_rows = 0 promises that no sequence has exactly one row (that launch is skipped), anything else
- * makes no promise.
+ * max_seqlen_q / max_seqlen_k: the most rows / keys any sequence has in this step (0 = unknown).  Three kernels
+ * share the work: sequences with several rows run on a bf16 MFMA tile kernel (head sizes in multiples of 16) sized from
+ * max_seqlen_q; sequences with one row on a decode kernel that reads K/V once per group of query heads and cuts long
+ * contexts into key slices (planned from max_seqlen_k, joined through `workspace`); whatever shape neither takes
+ * runs one row per wave.  single_rows = 0 promises that no sequence has exactly one row; max_seqlen_q = 1 that all do.
  */
 NV_API int nv_attn_scoremod_paged(const void* q, const void* k_cache, const void* v_cache, void* out,
                                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                                   const int32_t* block_tables, int num_seqs, int max_blocks_per_seq, int64_t T,
                                   int H, int G, int D, int Dv, int64_t num_blocks, int block_size, float scale,
                                   float softcap, const float* sink, const float* dist_bias, int n_dist,
-                                  int max_seqlen_q, int single_rows, int dtype, int64_t q_stride,
-                                  int64_t out_stride, void* stream);
+                                  int max_seqlen_q, int max_seqlen_k, int single_rows, int dtype, int64_t q_stride,
+                                  int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream);
+/* Scratch bytes the launch above needs for these sizes (key slices of single rows; 0 when it needs none). */
+NV_API int64_t nv_attn_scoremod_workspace_bytes(int num_seqs, int64_t T, int H, int G, int Dv, int max_seqlen_k);
 
 /*
  * Short causal convolution over time per channel, then SiLU, with the last taps-1 inputs of every sequence carried

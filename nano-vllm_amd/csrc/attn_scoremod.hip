@@ -17,6 +17,8 @@
 // (angle = position * inv_freq[i] as an fp32 product, full-precision sincosf), an optional position-dependent
 // query temperature q *= 1 + coef * ln(floor((p + 1) / every) + 1), and the scatter of the step's K/V rows into the
 // cache.
+#include <algorithm>
+
 #include "nv_common.h"
 #include "../../include/nanovllm_hip_mixers.h"
 
@@ -102,7 +104,8 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
     }
     const int b = lo;
     const int len_q = cu_q[b + 1] - cu_q[b], len_k = cu_k[b + 1] - cu_k[b];
-    if (only_single_rows && len_q != 1) return;          // the tile kernel has the sequences with several rows
+    // only_single_rows: 0 = every row, 1 = sequences with one row only, 2 = sequences with several rows only
+    if ((only_single_rows == 1 && len_q != 1) || (only_single_rows == 2 && len_q == 1)) return;
     const int pos = len_k - len_q + (t - cu_q[b]);      // this query's position; it sees keys 0 .. pos
     const int g = h / (H / G);
     for (int d = lane; d < D; d += 64) qs[d] = (float)q[(int64_t)t * q_stride + (int64_t)h * D + d];
@@ -235,7 +238,9 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
             *(uint4*)(ldsK + key * k_ld + 8 * ch) = val;
         }
         for (int c = tid; c < kTileK * vchunks; c += kTileThreads) {
-            const int key = c / vchunks, ch = c - key * vchunks, j = base + key;
+            // consecutive lanes take consecutive keys: the eight 2-byte stores below then land in consecutive LDS
+            // words (with the chunk index fastest they would all hit one bank)
+            const int key = c & (kTileK - 1), ch = c / kTileK, j = base + key;
             uint4 val = make_uint4(0, 0, 0, 0);
             if (j < len_k) {
                 const int64_t row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
@@ -328,6 +333,244 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------ single rows
+// Decode kernel: sequences with ONE row in the step.  A workgroup takes one (sequence, kv head) and one slice of
+// the keys, for all H / G query heads of the group at once, so K and V are read once per group.  Its four waves
+// split the slice; a wave walks its keys 64 at a time: lane j reads key j's row with 16-byte loads and scores it
+// against every head (q sits in LDS, read as broadcasts), the weights go through LDS, then the lanes turn to value
+// channels (two neighbouring channels per lane) and stream the tile's V rows.  No barrier inside the loop.  The
+// waves' running (max, sum, accumulator) are joined through LDS, and the slices through a workspace and a second
+// small launch that also puts the sink into the denominator.
+constexpr int kDecRep = 8;             // query heads per kv head handled at once (larger groups go round again)
+constexpr int kDecThreads = 256;
+constexpr int kDecDvPairs = 2;         // Dv <= 256: lane handles channels 2 * lane + 128 * i, i < 2
+
+template <typename T> struct Vec16;
+template <> struct Vec16<__bf16> { static constexpr int n = 8; };
+template <> struct Vec16<float> { static constexpr int n = 4; };
+
+template <typename T>
+__device__ __forceinline__ void load16(const T* p, float* o);
+template <>
+__device__ __forceinline__ void load16<__bf16>(const __bf16* p, float* o) {
+    const uint4 u = *(const uint4*)p;
+    o[0] = bf16_lo(u.x); o[1] = bf16_hi(u.x); o[2] = bf16_lo(u.y); o[3] = bf16_hi(u.y);
+    o[4] = bf16_lo(u.z); o[5] = bf16_hi(u.z); o[6] = bf16_lo(u.w); o[7] = bf16_hi(u.w);
+}
+template <>
+__device__ __forceinline__ void load16<float>(const float* p, float* o) {
+    const float4 u = *(const float4*)p;
+    o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
+}
+template <typename T>
+__device__ __forceinline__ void load_pair(const T* p, float& a, float& b);
+template <>
+__device__ __forceinline__ void load_pair<__bf16>(const __bf16* p, float& a, float& b) {
+    const uint32_t u = *(const uint32_t*)p;
+    a = bf16_lo(u); b = bf16_hi(u);
+}
+template <>
+__device__ __forceinline__ void load_pair<float>(const float* p, float& a, float& b) {
+    const float2 u = *(const float2*)p;
+    a = u.x; b = u.y;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
+    float* __restrict__ ws, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
+    const int* __restrict__ block_tables, int max_blocks, int H, int G, int D, int Dv, int block_size, float scale,
+    float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
+    int64_t out_stride, int splits, int slice_keys, int64_t T_rows) {
+    extern __shared__ float dsm[];
+    const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+    const int t = cu_q[b];
+    if (cu_q[b + 1] - t != 1) return;                        // rows of longer portions belong to the other kernels
+    const int n_keys = cu_k[b + 1] - cu_k[b], pos = n_keys - 1;
+    const int rep_all = H / G;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float* qs = dsm;                                          // [kDecRep][D]
+    float* ps = qs + kDecRep * D;                             // [4 waves][kDecRep][64]
+    float* red = ps + 4 * kDecRep * 64;                       // [4 waves][kDecRep][2 + Dv]
+    const int* table = block_tables + (int64_t)b * max_blocks;
+    const int k_lo = split * slice_keys, k_hi = min(n_keys, k_lo + slice_keys);
+    constexpr int VN = Vec16<T>::n;
+    for (int h0 = 0; h0 < rep_all; h0 += kDecRep) {
+        const int rep = min(kDecRep, rep_all - h0);
+        const int head0 = g * rep_all + h0;
+        __syncthreads();
+        for (int i = tid; i < rep * D; i += kDecThreads)
+            qs[i] = (float)q[(int64_t)t * q_stride + (int64_t)(head0 + i / D) * D + (i % D)];
+        __syncthreads();
+        float m[kDecRep], l[kDecRep], acc[kDecRep][2 * kDecDvPairs];
+#pragma unroll
+        for (int r = 0; r < kDecRep; ++r) {
+            m[r] = -INFINITY;
+            l[r] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 2 * kDecDvPairs; ++i) acc[r][i] = 0.f;
+        }
+        // the slice's 64-key tiles go round the four waves
+        for (int base = k_lo + wave * 64; base < k_hi; base += 4 * 64) {
+            const int j = base + lane;
+            const bool live = j < k_hi;
+            float sc[kDecRep];
+#pragma unroll
+            for (int r = 0; r < kDecRep; ++r) sc[r] = 0.f;
+            int64_t row = 0;
+            if (live) {
+                row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
+                const T* kr = k_cache + row * D;
+                for (int d = 0; d < D; d += VN) {
+                    float kv[VN];
+                    load16<T>(kr + d, kv);
+#pragma unroll
+                    for (int r = 0; r < kDecRep; ++r) {
+                        if (r < rep) {
+#pragma unroll
+                            for (int e = 0; e < VN; ++e) sc[r] += qs[r * D + d + e] * kv[e];
+                        }
+                    }
+                }
+            }
+            float* pw = ps + (wave * kDecRep) * 64;
+#pragma unroll
+            for (int r = 0; r < kDecRep; ++r) {
+                if (r < rep) {
+                    float x = -INFINITY;
+                    if (live) {
+                        x = sc[r] * scale;
+                        if (softcap > 0.f) x = softcap * tanhf(x / softcap);
+                        if (dist_bias) x += dist_bias[(int64_t)(head0 + r) * n_dist + min(pos - j, n_dist - 1)];
+                    }
+                    float tm = x;
+#pragma unroll
+                    for (int o = 32; o > 0; o >>= 1) tm = fmaxf(tm, __shfl_xor(tm, o));
+                    const float m_new = fmaxf(m[r], tm);          // finite: the tile has at least one live key
+                    const float p = live ? expf(x - m_new) : 0.f;
+                    const float corr = expf(m[r] - m_new);
+                    l[r] = l[r] * corr + wave_sum(p);
+                    m[r] = m_new;
+#pragma unroll
+                    for (int i = 0; i < 2 * kDecDvPairs; ++i) acc[r][i] *= corr;
+                    pw[r * 64 + lane] = p;
+                }
+            }
+            // rows of the tile's keys for the value pass (the wave's own LDS words: no workgroup barrier needed)
+            const int n_tile = min(64, k_hi - base);
+            for (int jj = 0; jj < n_tile; ++jj) {
+                const int64_t vrow = __shfl(row, jj);
+                const T* vr = v_cache + vrow * Dv;
+#pragma unroll
+                for (int i = 0; i < kDecDvPairs; ++i) {
+                    const int c = 2 * lane + 128 * i;
+                    if (c < Dv) {
+                        float va, vb;
+                        load_pair<T>(vr + c, va, vb);
+#pragma unroll
+                        for (int r = 0; r < kDecRep; ++r) {
+                            if (r < rep) {
+                                const float pj = pw[r * 64 + jj];
+                                acc[r][2 * i] += pj * va;
+                                acc[r][2 * i + 1] += pj * vb;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // ---- join the four waves ---------------------------------------------------------------------------
+        const int rs = 2 + Dv;
+#pragma unroll
+        for (int r = 0; r < kDecRep; ++r) {
+            if (r < rep) {
+                float* dst = red + ((wave * kDecRep) + r) * rs;
+                if (lane == 0) {
+                    dst[0] = m[r];
+                    dst[1] = l[r];
+                }
+#pragma unroll
+                for (int i = 0; i < kDecDvPairs; ++i) {
+                    const int c = 2 * lane + 128 * i;
+                    if (c < Dv) {
+                        dst[2 + c] = acc[r][2 * i];
+                        dst[2 + c + 1] = acc[r][2 * i + 1];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        for (int r = wave; r < rep; r += 4) {                 // wave w finishes heads w, w + 4, ...
+            float mm = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) mm = fmaxf(mm, red[(w * kDecRep + r) * rs]);
+            float ll = 0.f, f[4];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float mw = red[(w * kDecRep + r) * rs];
+                f[w] = mw == -INFINITY ? 0.f : expf(mw - mm);  // a wave (or the whole slice) may have had no keys
+                ll += f[w] * red[(w * kDecRep + r) * rs + 1];
+            }
+            const int head = head0 + r;
+            if (splits == 1) {
+                float den = ll, osc = 1.f;
+                if (sink) {
+                    const float sk = sink[head], m2 = fmaxf(mm, sk);
+                    osc = expf(mm - m2);
+                    den = ll * osc + expf(sk - m2);
+                }
+                for (int c = lane; c < Dv; c += 64) {
+                    float o = 0.f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) o += f[w] * red[(w * kDecRep + r) * rs + 2 + c];
+                    out[(int64_t)t * out_stride + (int64_t)head * Dv + c] = (T)(o * osc / den);
+                }
+            } else {
+                float* wrow = ws + (((int64_t)split * T_rows + t) * H + head) * rs;
+                if (lane == 0) {
+                    wrow[0] = mm;
+                    wrow[1] = ll;
+                }
+                for (int c = lane; c < Dv; c += 64) {
+                    float o = 0.f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) o += f[w] * red[(w * kDecRep + r) * rs + 2 + c];
+                    wrow[2 + c] = o;
+                }
+            }
+        }
+    }
+}
+
+// Joins the key slices of a single row: one wave per (sequence, head).
+template <typename T>
+__global__ __launch_bounds__(64) void attn_scoremod_decode_merge_kernel(
+    const float* __restrict__ ws, T* __restrict__ out, const int* __restrict__ cu_q, const float* __restrict__ sink,
+    int H, int Dv, int64_t out_stride, int splits, int64_t T_rows) {
+    const int b = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int t = cu_q[b];
+    if (cu_q[b + 1] - t != 1) return;
+    const int rs = 2 + Dv;
+    float mm = -INFINITY;
+    for (int s = 0; s < splits; ++s) mm = fmaxf(mm, ws[(((int64_t)s * T_rows + t) * H + head) * rs]);
+    float m2 = mm;
+    if (sink) m2 = fmaxf(mm, sink[head]);
+    float den = sink ? expf(sink[head] - m2) : 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float* w = ws + (((int64_t)s * T_rows + t) * H + head) * rs;
+        if (w[0] != -INFINITY) den += expf(w[0] - m2) * w[1];
+    }
+    for (int c = lane; c < Dv; c += 64) {
+        float o = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float* w = ws + (((int64_t)s * T_rows + t) * H + head) * rs;
+            if (w[0] != -INFINITY) o += expf(w[0] - m2) * w[2 + c];
+        }
+        out[(int64_t)t * out_stride + (int64_t)head * Dv + c] = (T)(o / den);
+    }
+}
+
 }  // namespace nv
 
 extern "C" int nv_qk_prep_store(const void* q, const void* k, const void* v, void* q_out, void* k_cache,
@@ -359,12 +602,38 @@ extern "C" int nv_qk_prep_store(const void* q, const void* k, const void* v, voi
     return check_launch("nv_qk_prep_store");
 }
 
+namespace nv {
+struct DecodePlan {
+    int splits, slice_keys;
+    int64_t ws_bytes;
+};
+// Key slices of the decode kernel: about four workgroups per CU, and never less than 64 keys per wave of a slice.
+static DecodePlan decode_plan(int num_seqs, int64_t T, int H, int G, int Dv, int max_seqlen_k) {
+    DecodePlan p{1, 0, 0};
+    const int64_t blocks = (int64_t)num_seqs * G;
+    if (max_seqlen_k > 0 && blocks > 0) {
+        const int64_t want = (1024 + blocks - 1) / blocks, most = std::max(1, max_seqlen_k / 256);
+        p.splits = (int)std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 64));
+    }
+    const int len = max_seqlen_k > 0 ? max_seqlen_k : (1 << 30);
+    p.slice_keys = ((len + p.splits - 1) / p.splits + 63) / 64 * 64;
+    p.ws_bytes = p.splits > 1 ? (int64_t)p.splits * T * H * (2 + Dv) * (int64_t)sizeof(float) : 0;
+    return p;
+}
+}  // namespace nv
+
+extern "C" int64_t nv_attn_scoremod_workspace_bytes(int num_seqs, int64_t T, int H, int G, int Dv, int max_seqlen_k) {
+    if (num_seqs <= 0 || T <= 0 || H <= 0 || G <= 0 || Dv <= 0) return 0;
+    return nv::decode_plan(num_seqs, T, H, G, Dv, max_seqlen_k).ws_bytes;
+}
+
 extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const void* v_cache, void* out,
                                       const int* cu_seqlens_q, const int* cu_seqlens_k, const int* block_tables,
                                       int num_seqs, int max_blocks_per_seq, int64_t T, int H, int G, int D, int Dv,
                                       int64_t num_blocks, int block_size, float scale, float softcap,
                                       const float* sink, const float* dist_bias, int n_dist, int max_seqlen_q,
-                                      int single_rows, int dtype, int64_t q_stride, int64_t out_stride, void* stream) {
+                                      int max_seqlen_k, int single_rows, int dtype, int64_t q_stride,
+                                      int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream) {
     using namespace nv;
     NV_REQUIRE(num_seqs >= 0 && T >= 0 && H > 0 && G > 0 && D > 0 && Dv > 0 && block_size > 0 && num_blocks > 0 &&
                    max_blocks_per_seq > 0,
@@ -378,16 +647,23 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     NV_REQUIRE(D <= 1024, NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: D=%d exceeds 1024", D);
     NV_REQUIRE(!dist_bias || n_dist > 0, NV_ERR_INVALID_ARG, "nv_attn_scoremod_paged: bias without rows");
     NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_attn_scoremod_paged: bad dtype");
-    NV_REQUIRE(T < (1LL << 31) && H < 65536, NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: launch too large");
+    NV_REQUIRE(T < (1LL << 31) && H < 65536 && G < 65536, NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: launch too large");
     hipStream_t s = (hipStream_t)stream;
-    // Sequences with several rows go to the MFMA tile kernel when the shapes allow (bf16, head sizes in multiples of
-    // 16 up to 256, tiles within 64 KiB of LDS, 16-byte aligned rows); the row-wave kernel then takes the single rows
-    // only.  max_seqlen_q <= 0 (unknown) or 1 keeps everything on the row-wave kernel.
-    int only_single = 0;
+    const bool bf = dtype == NV_DTYPE_BF16;
+    const bool several = max_seqlen_q != 1, singles = single_rows != 0;      // what the step may hold
+    // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes in multiples of 16 up
+    // to 256, tiles within 64 KiB of LDS, aligned rows), else the row-per-wave kernel.
     const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 8) + (size_t)Dv * (kTileK + 8));
-    if (dtype == NV_DTYPE_BF16 && max_seqlen_q > 1 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 &&
-        tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
-        ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0) {
+    const bool tile_ok = bf && max_seqlen_q > 1 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 &&
+                         tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
+                         ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
+    // Sequences with one row: the decode kernel (key slices, the query heads of a group together) when rows can be
+    // read in 16-byte pieces, else the row-per-wave kernel.
+    const int vn = bf ? 8 : 4;
+    const size_t dec_lds = sizeof(float) * ((size_t)kDecRep * D + 4 * kDecRep * 64 + 4 * kDecRep * (2 + Dv));
+    const bool dec_ok = singles && D % vn == 0 && Dv % 2 == 0 && Dv <= 128 * kDecDvPairs && dec_lds <= 64 * 1024 &&
+                        ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
+    if (several && tile_ok) {
         const int tiles = (max_seqlen_q + kTileQ - 1) / kTileQ;
         NV_REQUIRE((int64_t)num_seqs * tiles < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: launch too large");
         const dim3 tgrid((unsigned)(num_seqs * tiles), (unsigned)H);
@@ -402,20 +678,49 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
 #undef NV_TILE_ARGS
         const int rc = check_launch("nv_attn_scoremod_paged (tile kernel)");
         if (rc != NV_OK) return rc;
-        if (single_rows == 0) return NV_OK;
-        only_single = 1;
     }
+    if (dec_ok) {
+        const DecodePlan plan = decode_plan(num_seqs, T, H, G, Dv, max_seqlen_k);
+        NV_REQUIRE(plan.ws_bytes == 0 || (workspace && workspace_bytes >= plan.ws_bytes), NV_ERR_WORKSPACE,
+                   "nv_attn_scoremod_paged: workspace of %lld bytes, need %lld", (long long)workspace_bytes,
+                   (long long)plan.ws_bytes);
+        const dim3 dgrid((unsigned)num_seqs, (unsigned)G, (unsigned)plan.splits);
+#define NV_DEC_ARGS(TT)                                                                                              \
+    (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, (TT*)out, (float*)workspace, cu_seqlens_q, cu_seqlens_k, \
+        block_tables, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,        \
+        q_stride, out_stride, plan.splits, plan.slice_keys, T
+        if (bf) hipLaunchKernelGGL(attn_scoremod_decode_kernel<__bf16>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(__bf16));
+        else hipLaunchKernelGGL(attn_scoremod_decode_kernel<float>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(float));
+#undef NV_DEC_ARGS
+        int rc = check_launch("nv_attn_scoremod_paged (decode kernel)");
+        if (rc != NV_OK) return rc;
+        if (plan.splits > 1) {
+            const dim3 mgrid((unsigned)num_seqs, (unsigned)H);
+            if (bf)
+                hipLaunchKernelGGL(attn_scoremod_decode_merge_kernel<__bf16>, mgrid, dim3(64), 0, s, (const float*)workspace,
+                                   (__bf16*)out, cu_seqlens_q, sink, H, Dv, out_stride, plan.splits, T);
+            else
+                hipLaunchKernelGGL(attn_scoremod_decode_merge_kernel<float>, mgrid, dim3(64), 0, s, (const float*)workspace,
+                                   (float*)out, cu_seqlens_q, sink, H, Dv, out_stride, plan.splits, T);
+            rc = check_launch("nv_attn_scoremod_paged (decode merge)");
+            if (rc != NV_OK) return rc;
+        }
+    }
+    // what is left for the row-per-wave kernel: 0 = every row, 1 = single rows only, 2 = longer portions only
+    const bool rw_several = several && !tile_ok, rw_singles = singles && !dec_ok;
+    if (!rw_several && !rw_singles) return NV_OK;
+    const int only = rw_several && rw_singles ? 0 : rw_singles ? 1 : 2;
     const size_t smem = sizeof(float) * (D + 64 + (D & 1)) + sizeof(int64_t) * 64;
     const dim3 grid((unsigned)T, (unsigned)H);
-    if (dtype == NV_DTYPE_BF16)
+    if (bf)
         hipLaunchKernelGGL(attn_scoremod_rowwave_kernel<__bf16>, grid, dim3(64), smem, s, (const __bf16*)q,
                            (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q, cu_seqlens_k,
                            block_tables, num_seqs, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink,
-                           dist_bias, n_dist, q_stride, out_stride, only_single);
+                           dist_bias, n_dist, q_stride, out_stride, only);
     else
         hipLaunchKernelGGL(attn_scoremod_rowwave_kernel<float>, grid, dim3(64), smem, s, (const float*)q,
                            (const float*)k_cache, (const float*)v_cache, (float*)out, cu_seqlens_q, cu_seqlens_k,
                            block_tables, num_seqs, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink,
-                           dist_bias, n_dist, q_stride, out_stride, only_single);
+                           dist_bias, n_dist, q_stride, out_stride, only);
     return check_launch("nv_attn_scoremod_paged");
 }

@@ -492,11 +492,14 @@ def attn_scoremod_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
         n_dist = dist_bias.shape[1]
     out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
     dll = _lib.mixers()
+    need = dll.nv_attn_scoremod_workspace_bytes(B, T, H, G, Dv, int(max_seqlen_k))
+    ws = _workspace(q.device, need) if need else None
     rc = dll.nv_attn_scoremod_paged(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
                                     cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), block_tables.data_ptr(), B,
                                     block_tables.shape[1], T, H, G, D, Dv, nb, bs, float(scale), float(softcap or 0.0),
                                     _f32c(sink, "sink") or None, _f32c(dist_bias, "dist_bias") or None, n_dist,
-                                    int(max_seqlen_q), int(single_rows), dt, q.stride(0), out.stride(0), _stream(q))
+                                    int(max_seqlen_q), int(max_seqlen_k), int(single_rows), dt, q.stride(0),
+                                    out.stride(0), _ptr(ws), ws.numel() if ws is not None else 0, _stream(q))
     _lib.check(rc, "nv_attn_scoremod_paged", dll)
     return out
 

@@ -158,6 +158,38 @@ def test_scoremod_attention_long_portions_cross_query_and_key_tiles(dtype, shape
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(8, 2, 96, 96), (16, 2, 64, 128), (12, 1, 32, 48), (3, 3, 20, 6), (4, 2, 128, 256)])
+@pytest.mark.parametrize("lens", [[1500, 700, 1, 64, 65], [300] * 40])
+def test_scoremod_attention_single_rows_key_slices_and_head_groups(dtype, shape, lens):
+    """Pure decode steps: long contexts cut into key slices (some slices of the shorter sequences are empty), one
+    key only, contexts of exactly one tile and one more, groups of 8 and 12 query heads per kv head, a head size
+    that is no multiple of a 16-byte piece, and a batch large enough that nothing is sliced."""
+    H, G, D, Dv = shape
+    bs = 24
+    nb = sum(-(-n // bs) for n in lens) + 2
+    a, r = _attention_pair(H, G, D, Dv, scale=D ** -0.5, softcap=25.0, temp_coef=0.3, temp_every=100, use_sink=True)
+    g = torch.Generator(device=DEV).manual_seed(9)
+    table = torch.randn(H, 200, generator=g, device=DEV)
+    a.set_distance_bias(table)
+    r.set_distance_bias(table)
+    with torch.no_grad():
+        a.sink.copy_(torch.randn(H, generator=g, device=DEV) * 2)
+        r.sink.copy_(a.sink)
+    ctx, pos = _context([1] * len(lens), lens, bs, nb, seed=5)
+    ctx.num_decode_seqs = len(lens)
+    T = len(lens)
+    mk = lambda *s: torch.randn(*s, generator=g, device=DEV).to(dtype)
+    kc, vc = mk(nb, bs, G, D), mk(nb, bs, G, Dv)
+    kc_r, vc_r = kc.clone(), vc.clone()
+    q, k, v = mk(T, H, D), mk(T, G, D), mk(T, G, Dv)
+    nv.set_context(ctx)
+    o = a(q, k, v, pos, kc, vc)
+    o_r = r(q, k, v, pos, kc_r, vc_r)
+    nv.set_context(None)
+    torch.testing.assert_close(o.float(), o_r.float(), **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 3, 4])
 def test_short_conv_in_portions_matches_one_pass(dtype, taps):
     C, slots_n = 200, 5
