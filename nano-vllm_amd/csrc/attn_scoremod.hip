@@ -186,8 +186,8 @@ __device__ __forceinline__ float fast_tanh(float x) {
     return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f);
 }
 
-template <int NS>     // NS: most 16-wide steps over D and over Dv (D, Dv <= 16 * NS)
-__global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
+template <int DS, int DVS>     // D = 16 DS, Dv = 16 DVS: every loop below has a compile-time length
+__global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
     __bf16* __restrict__ out, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int tiles_per_seq, int H, int G, int D, int Dv,
@@ -198,7 +198,6 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
     const int q0 = cu_q[b], len_q = cu_q[b + 1] - q0, len_k = cu_k[b + 1] - cu_k[b];
     if (len_q <= 1 || qt * kTileQ >= len_q) return;          // single rows belong to the row-wave kernel
     const int g = h / (H / G);
-    const int ds = D / 16, dvs = Dv / 16;
     const int k_ld = D + 8, v_ld = kTileK + 8;                // LDS row lengths in elements (16-byte multiples)
     __bf16* ldsK = (__bf16*)lds_raw;                          // [64][D + 8]
     __bf16* ldsV = ldsK + kTileK * k_ld;                      // [Dv][64 + 8]
@@ -211,46 +210,56 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
     const int wave_last_pos = start + min(row0 + 15, len_q - 1);
     const bool wave_live = row0 < len_q;
     // Q^T fragments: lane holds q[my_row][16 s + 4 lg .. + 3]
-    s16x4 qf[NS];
+    s16x4 qf[DS];
     {
         const __bf16* qr = q + (int64_t)(q0 + my_row) * q_stride + (int64_t)h * D;
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
-            qf[s] = s < ds ? *(const s16x4*)(qr + 16 * s + 4 * lg) : s16x4{0, 0, 0, 0};
+        for (int s = 0; s < DS; ++s) qf[s] = *(const s16x4*)(qr + 16 * s + 4 * lg);
     }
-    f32x4 oacc[NS];
+    f32x4 oacc[DVS];
 #pragma unroll
-    for (int i = 0; i < NS; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < DVS; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
     const int* table = block_tables + (int64_t)b * max_blocks;
     const float* bias_h = dist_bias ? dist_bias + (int64_t)h * n_dist : nullptr;
     const int last_pos = start + min(qt * kTileQ + kTileQ, len_q) - 1;      // the tile's last query sees keys 0 .. last_pos
-    const int kchunks = D / 8, vchunks = Dv / 8;
+    // Loading a tile: thread (key = tid % 64, quarter = tid / 64) fetches 16-byte pieces quarter, quarter + 4, ... of
+    // its key's K row and V row.  One block-table lookup per thread and tile, every load of a tile issued before
+    // anything waits on one, and the next tile's loads are in flight while this tile is computed.
+    const int my_key = tid & (kTileK - 1), my_quarter = tid >> 6;
+    constexpr int KP = DS / 2, VP = DVS / 2;                    // 16-byte pieces per thread of a K row / a V row
+    uint4 kreg[KP], vreg[VP];
+    auto fetch = [&](int base) {
+        const int j = base + my_key;
+        const bool in = j < len_k;
+        int64_t row = 0;
+        if (in) row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
+#pragma unroll
+        for (int i = 0; i < KP; ++i)
+            kreg[i] = in ? *(const uint4*)(k_cache + row * D + 8 * (my_quarter + 4 * i)) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < VP; ++i)
+            vreg[i] = in ? *(const uint4*)(v_cache + row * Dv + 8 * (my_quarter + 4 * i)) : make_uint4(0, 0, 0, 0);
+    };
+    fetch(0);
     for (int base = 0; base <= last_pos; base += kTileK) {
         __syncthreads();                                      // the previous tile has been consumed
-        for (int c = tid; c < kTileK * kchunks; c += kTileThreads) {
-            const int key = c / kchunks, ch = c - key * kchunks, j = base + key;
-            uint4 val = make_uint4(0, 0, 0, 0);
-            if (j < len_k) {
-                const int64_t row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
-                val = *(const uint4*)(k_cache + row * D + 8 * ch);
-            }
-            *(uint4*)(ldsK + key * k_ld + 8 * ch) = val;
-        }
-        for (int c = tid; c < kTileK * vchunks; c += kTileThreads) {
-            // consecutive lanes take consecutive keys: the eight 2-byte stores below then land in consecutive LDS
-            // words (with the chunk index fastest they would all hit one bank)
-            const int key = c & (kTileK - 1), ch = c / kTileK, j = base + key;
-            uint4 val = make_uint4(0, 0, 0, 0);
-            if (j < len_k) {
-                const int64_t row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
-                val = *(const uint4*)(v_cache + row * Dv + 8 * ch);
-            }
-            const unsigned short* e = (const unsigned short*)&val;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ((unsigned short*)ldsV)[(8 * ch + i) * v_ld + key] = e[i];
+        for (int i = 0; i < KP; ++i) *(uint4*)(ldsK + my_key * k_ld + 8 * (my_quarter + 4 * i)) = kreg[i];
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            // V goes in transposed; consecutive lanes hold consecutive keys, so each of the eight 2-byte stores of a
+            // wave lands in consecutive LDS words
+            const int ch = my_quarter + 4 * i;
+            const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                ((unsigned short*)ldsV)[(8 * ch + 2 * e) * v_ld + my_key] = (unsigned short)(w[e] & 0xffffu);
+                ((unsigned short*)ldsV)[(8 * ch + 2 * e + 1) * v_ld + my_key] = (unsigned short)(w[e] >> 16);
+            }
         }
         __syncthreads();
+        if (base + kTileK <= last_pos) fetch(base + kTileK);
         if (!wave_live || base > wave_last_pos) continue;     // (uniform per wave; the barriers above stay matched)
         // ---- S^T for four 16-key blocks -----------------------------------------------------------------------
         f32x4 sacc[4];
@@ -258,11 +267,9 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
         for (int kb = 0; kb < 4; ++kb) {
             sacc[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                if (s < ds) {
-                    const s16x4 a = *(const s16x4*)(ldsK + (kb * 16 + lq) * k_ld + 16 * s + 4 * lg);
-                    sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sacc[kb], 0, 0, 0);
-                }
+            for (int s = 0; s < DS; ++s) {
+                const s16x4 a = *(const s16x4*)(ldsK + (kb * 16 + lq) * k_ld + 16 * s + 4 * lg);
+                sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qf[s], sacc[kb], 0, 0, 0);
             }
         }
         // ---- modifiers, mask, running maximum -----------------------------------------------------------------
@@ -287,7 +294,7 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
         m = m_new;
         l *= corr;
 #pragma unroll
-        for (int i = 0; i < NS; ++i) oacc[i] *= corr;
+        for (int i = 0; i < DVS; ++i) oacc[i] *= corr;
         // ---- P^T, then O^T += V^T P^T ---------------------------------------------------------------------------
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
@@ -300,11 +307,9 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
             const uint32_t p01 = pack_bf16(p[0], p[1]), p23 = pack_bf16(p[2], p[3]);
             const s16x4 pb = __builtin_bit_cast(s16x4, make_uint2(p01, p23));
 #pragma unroll
-            for (int dv = 0; dv < NS; ++dv) {
-                if (dv < dvs) {
-                    const s16x4 a = *(const s16x4*)(ldsV + (dv * 16 + lq) * v_ld + kb * 16 + 4 * lg);
-                    oacc[dv] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dv], 0, 0, 0);
-                }
+            for (int dv = 0; dv < DVS; ++dv) {
+                const s16x4 a = *(const s16x4*)(ldsV + (dv * 16 + lq) * v_ld + kb * 16 + 4 * lg);
+                oacc[dv] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dv], 0, 0, 0);
             }
         }
     }
@@ -317,18 +322,16 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
         const float corr = __expf(m - m_new);
         l = l * corr + __expf(sk - m_new);
 #pragma unroll
-        for (int i = 0; i < NS; ++i) oacc[i] *= corr;
+        for (int i = 0; i < DVS; ++i) oacc[i] *= corr;
     }
     if (row0 + lq < len_q) {
         const float inv = 1.0f / l;
         __bf16* orow = out + (int64_t)(q0 + row0 + lq) * out_stride + (int64_t)h * Dv;
 #pragma unroll
-        for (int dv = 0; dv < NS; ++dv) {
-            if (dv < dvs) {
-                const uint2 pk = make_uint2(pack_bf16(oacc[dv][0] * inv, oacc[dv][1] * inv),
-                                            pack_bf16(oacc[dv][2] * inv, oacc[dv][3] * inv));
-                *(uint2*)(orow + dv * 16 + 4 * lg) = pk;
-            }
+        for (int dv = 0; dv < DVS; ++dv) {
+            const uint2 pk = make_uint2(pack_bf16(oacc[dv][0] * inv, oacc[dv][1] * inv),
+                                        pack_bf16(oacc[dv][2] * inv, oacc[dv][3] * inv));
+            *(uint2*)(orow + dv * 16 + 4 * lg) = pk;
         }
     }
 }
@@ -338,13 +341,13 @@ __global__ __launch_bounds__(kTileThreads) void attn_scoremod_tile_kernel(
 // Decode kernel: sequences with ONE row in the step.  A workgroup takes one (sequence, kv head) and one slice of
 // the keys, for all H / G query heads of the group at once, so K and V are read once per group.  Its four waves
 // split the slice; a wave walks its keys 64 at a time: lane j reads key j's row with 16-byte loads and scores it
-// against every head (q sits in LDS, read as broadcasts), the weights go through LDS, then the lanes turn to value
-// channels (two neighbouring channels per lane) and stream the tile's V rows.  No barrier inside the loop.  The
+// against every head (q sits in LDS, read as broadcasts), the weights go through LDS, then the lanes regroup for the
+// value pass: a V row is cut into 16-byte pieces and the wave's load instruction covers several whole rows, each lane
+// keeping one piece of every head's accumulator.  No barrier inside the loop.  The
 // waves' running (max, sum, accumulator) are joined through LDS, and the slices through a workspace and a second
 // small launch that also puts the sink into the denominator.
 constexpr int kDecRep = 8;             // query heads per kv head handled at once (larger groups go round again)
 constexpr int kDecThreads = 256;
-constexpr int kDecDvPairs = 2;         // Dv <= 256: lane handles channels 2 * lane + 128 * i, i < 2
 
 template <typename T> struct Vec16;
 template <> struct Vec16<__bf16> { static constexpr int n = 8; };
@@ -364,25 +367,12 @@ __device__ __forceinline__ void load16<float>(const float* p, float* o) {
     o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
 }
 template <typename T>
-__device__ __forceinline__ void load_pair(const T* p, float& a, float& b);
-template <>
-__device__ __forceinline__ void load_pair<__bf16>(const __bf16* p, float& a, float& b) {
-    const uint32_t u = *(const uint32_t*)p;
-    a = bf16_lo(u); b = bf16_hi(u);
-}
-template <>
-__device__ __forceinline__ void load_pair<float>(const float* p, float& a, float& b) {
-    const float2 u = *(const float2*)p;
-    a = u.x; b = u.y;
-}
-
-template <typename T>
 __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     float* __restrict__ ws, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int D, int Dv, int block_size, float scale,
     float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride, int splits, int slice_keys, int64_t T_rows) {
+    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2) {
     extern __shared__ float dsm[];
     const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
     const int t = cu_q[b];
@@ -390,12 +380,18 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     const int n_keys = cu_k[b + 1] - cu_k[b], pos = n_keys - 1;
     const int rep_all = H / G;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int VN = Vec16<T>::n;
+    const int rs = 2 + Dv;
     float* qs = dsm;                                          // [kDecRep][D]
     float* ps = qs + kDecRep * D;                             // [4 waves][kDecRep][64]
     float* red = ps + 4 * kDecRep * 64;                       // [4 waves][kDecRep][2 + Dv]
+    int64_t* rws = (int64_t*)(red + 4 * kDecRep * rs + ((4 * kDecRep * rs + kDecRep * D) & 1));   // [4 waves][64] rows
     const int* table = block_tables + (int64_t)b * max_blocks;
     const int k_lo = split * slice_keys, k_hi = min(n_keys, k_lo + slice_keys);
-    constexpr int VN = Vec16<T>::n;
+    // value pass: a V row is cut into 16-byte pieces; lane (sub, piece) = (lane >> cpr_log2, lane & (2^cpr_log2 - 1))
+    // takes piece `piece` of every (64 >> cpr_log2)-th key, so one load instruction of the wave covers several whole rows
+    const int piece = lane & ((1 << cpr_log2) - 1), sub = lane >> cpr_log2, rows_per_load = 64 >> cpr_log2;
+    const bool piece_live = piece * VN < Dv;
     for (int h0 = 0; h0 < rep_all; h0 += kDecRep) {
         const int rep = min(kDecRep, rep_all - h0);
         const int head0 = g * rep_all + h0;
@@ -403,14 +399,16 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
         for (int i = tid; i < rep * D; i += kDecThreads)
             qs[i] = (float)q[(int64_t)t * q_stride + (int64_t)(head0 + i / D) * D + (i % D)];
         __syncthreads();
-        float m[kDecRep], l[kDecRep], acc[kDecRep][2 * kDecDvPairs];
+        float m[kDecRep], l[kDecRep], acc[kDecRep][VN];
 #pragma unroll
         for (int r = 0; r < kDecRep; ++r) {
             m[r] = -INFINITY;
             l[r] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 2 * kDecDvPairs; ++i) acc[r][i] = 0.f;
+            for (int i = 0; i < VN; ++i) acc[r][i] = 0.f;
         }
+        float* pw = ps + (wave * kDecRep) * 64;
+        int64_t* rw = rws + wave * 64;
         // the slice's 64-key tiles go round the four waves
         for (int base = k_lo + wave * 64; base < k_hi; base += 4 * 64) {
             const int j = base + lane;
@@ -422,7 +420,8 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
             if (live) {
                 row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
                 const T* kr = k_cache + row * D;
-                for (int d = 0; d < D; d += VN) {
+#pragma unroll 8
+                for (int d = 0; d < D; d += VN) {             // unrolled: eight 16-byte loads in flight per lane
                     float kv[VN];
                     load16<T>(kr + d, kv);
 #pragma unroll
@@ -434,9 +433,11 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                     }
                 }
             }
-            float* pw = ps + (wave * kDecRep) * 64;
+            rw[lane] = row;
+            float corr[kDecRep];
 #pragma unroll
             for (int r = 0; r < kDecRep; ++r) {
+                corr[r] = 1.f;
                 if (r < rep) {
                     float x = -INFINITY;
                     if (live) {
@@ -449,54 +450,48 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                     for (int o = 32; o > 0; o >>= 1) tm = fmaxf(tm, __shfl_xor(tm, o));
                     const float m_new = fmaxf(m[r], tm);          // finite: the tile has at least one live key
                     const float p = live ? expf(x - m_new) : 0.f;
-                    const float corr = expf(m[r] - m_new);
-                    l[r] = l[r] * corr + wave_sum(p);
+                    corr[r] = expf(m[r] - m_new);
+                    l[r] = l[r] * corr[r] + wave_sum(p);
                     m[r] = m_new;
-#pragma unroll
-                    for (int i = 0; i < 2 * kDecDvPairs; ++i) acc[r][i] *= corr;
                     pw[r * 64 + lane] = p;
+#pragma unroll
+                    for (int i = 0; i < VN; ++i) acc[r][i] *= corr[r];
                 }
             }
-            // rows of the tile's keys for the value pass (the wave's own LDS words: no workgroup barrier needed)
-            const int n_tile = min(64, k_hi - base);
-            for (int jj = 0; jj < n_tile; ++jj) {
-                const int64_t vrow = __shfl(row, jj);
-                const T* vr = v_cache + vrow * Dv;
+            // the tile's V rows (the wave reads its own LDS words: no workgroup barrier needed); keys past the slice
+            // have weight 0 and row 0, which is a row of the cache like any other
+            if (piece_live) {
+#pragma unroll 4
+                for (int jj = sub; jj < 64; jj += rows_per_load) {
+                    float vv[VN];
+                    load16<T>(v_cache + rw[jj] * Dv + piece * VN, vv);
 #pragma unroll
-                for (int i = 0; i < kDecDvPairs; ++i) {
-                    const int c = 2 * lane + 128 * i;
-                    if (c < Dv) {
-                        float va, vb;
-                        load_pair<T>(vr + c, va, vb);
+                    for (int r = 0; r < kDecRep; ++r) {
+                        if (r < rep) {
+                            const float pj = pw[r * 64 + jj];
 #pragma unroll
-                        for (int r = 0; r < kDecRep; ++r) {
-                            if (r < rep) {
-                                const float pj = pw[r * 64 + jj];
-                                acc[r][2 * i] += pj * va;
-                                acc[r][2 * i + 1] += pj * vb;
-                            }
+                            for (int e = 0; e < VN; ++e) acc[r][e] += pj * vv[e];
                         }
                     }
                 }
             }
         }
-        // ---- join the four waves ---------------------------------------------------------------------------
-        const int rs = 2 + Dv;
+        // ---- join the lanes that share a piece, then the four waves ---------------------------------------------
 #pragma unroll
         for (int r = 0; r < kDecRep; ++r) {
             if (r < rep) {
+                for (int o = 1 << cpr_log2; o < 64; o <<= 1) {
+#pragma unroll
+                    for (int e = 0; e < VN; ++e) acc[r][e] += __shfl_xor(acc[r][e], o);
+                }
                 float* dst = red + ((wave * kDecRep) + r) * rs;
                 if (lane == 0) {
                     dst[0] = m[r];
                     dst[1] = l[r];
                 }
+                if (sub == 0 && piece_live) {
 #pragma unroll
-                for (int i = 0; i < kDecDvPairs; ++i) {
-                    const int c = 2 * lane + 128 * i;
-                    if (c < Dv) {
-                        dst[2 + c] = acc[r][2 * i];
-                        dst[2 + c + 1] = acc[r][2 * i + 1];
-                    }
+                    for (int e = 0; e < VN; ++e) dst[2 + piece * VN + e] = acc[r][e];
                 }
             }
         }
@@ -651,17 +646,19 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     hipStream_t s = (hipStream_t)stream;
     const bool bf = dtype == NV_DTYPE_BF16;
     const bool several = max_seqlen_q != 1, singles = single_rows != 0;      // what the step may hold
-    // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes in multiples of 16 up
-    // to 256, tiles within 64 KiB of LDS, aligned rows), else the row-per-wave kernel.
+    // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes 32, 64, 96 or 128, aligned rows), else the row-per-wave kernel.
     const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 8) + (size_t)Dv * (kTileK + 8));
-    const bool tile_ok = bf && max_seqlen_q > 1 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 &&
-                         tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
+    const auto tile_size = [](int n) { return n == 32 || n == 64 || n == 96 || n == 128; };      // built tile shapes
+    const bool tile_ok = bf && max_seqlen_q > 1 && tile_size(D) && tile_size(Dv) && tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
                          ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
     // Sequences with one row: the decode kernel (key slices, the query heads of a group together) when rows can be
     // read in 16-byte pieces, else the row-per-wave kernel.
     const int vn = bf ? 8 : 4;
-    const size_t dec_lds = sizeof(float) * ((size_t)kDecRep * D + 4 * kDecRep * 64 + 4 * kDecRep * (2 + Dv));
-    const bool dec_ok = singles && D % vn == 0 && Dv % 2 == 0 && Dv <= 128 * kDecDvPairs && dec_lds <= 64 * 1024 &&
+    const size_t dec_lds = sizeof(float) * ((size_t)kDecRep * D + 4 * kDecRep * 64 + 4 * kDecRep * (2 + Dv) + 1) +
+                           sizeof(int64_t) * 4 * 64;
+    int cpr_log2 = 0;                                          // 16-byte pieces per V row, rounded up to a power of two
+    while ((vn << cpr_log2) < Dv) ++cpr_log2;
+    const bool dec_ok = singles && D % vn == 0 && Dv % vn == 0 && cpr_log2 <= 6 && dec_lds <= 64 * 1024 &&
                         ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
     if (several && tile_ok) {
         const int tiles = (max_seqlen_q + kTileQ - 1) / kTileQ;
@@ -671,10 +668,13 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     (const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q, cu_seqlens_k,      \
         block_tables, max_blocks_per_seq, tiles, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,  \
         q_stride, out_stride
-        if (D <= 128 && Dv <= 128)
-            hipLaunchKernelGGL(attn_scoremod_tile_kernel<8>, tgrid, dim3(kTileThreads), tile_lds, s, NV_TILE_ARGS);
-        else
-            hipLaunchKernelGGL(attn_scoremod_tile_kernel<16>, tgrid, dim3(kTileThreads), tile_lds, s, NV_TILE_ARGS);
+#define NV_TILE_CASE(A, B)                                                                                          \
+    if (D == 16 * A && Dv == 16 * B)                                                                                \
+        hipLaunchKernelGGL((attn_scoremod_tile_kernel<A, B>), tgrid, dim3(kTileThreads), tile_lds, s, NV_TILE_ARGS);
+#define NV_TILE_ROW(A) NV_TILE_CASE(A, 2) NV_TILE_CASE(A, 4) NV_TILE_CASE(A, 6) NV_TILE_CASE(A, 8)
+        NV_TILE_ROW(2) NV_TILE_ROW(4) NV_TILE_ROW(6) NV_TILE_ROW(8)
+#undef NV_TILE_ROW
+#undef NV_TILE_CASE
 #undef NV_TILE_ARGS
         const int rc = check_launch("nv_attn_scoremod_paged (tile kernel)");
         if (rc != NV_OK) return rc;
@@ -688,7 +688,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
 #define NV_DEC_ARGS(TT)                                                                                              \
     (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, (TT*)out, (float*)workspace, cu_seqlens_q, cu_seqlens_k, \
         block_tables, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,        \
-        q_stride, out_stride, plan.splits, plan.slice_keys, T
+        q_stride, out_stride, plan.splits, plan.slice_keys, T, cpr_log2
         if (bf) hipLaunchKernelGGL(attn_scoremod_decode_kernel<__bf16>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(__bf16));
         else hipLaunchKernelGGL(attn_scoremod_decode_kernel<float>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(float));
 #undef NV_DEC_ARGS

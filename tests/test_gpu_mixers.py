@@ -77,6 +77,9 @@ def test_gelu_tanh_and_mul(dtype):
     g = torch.Generator(device=DEV).manual_seed(1)
     x = (3 * torch.randn(19, 2 * 72 + 6, generator=g, device=DEV)).to(dtype)[:, :2 * 72]
     torch.testing.assert_close(activation.GeluTanhAndMul()(x).float(), ref.GeluTanhAndMul()(x).float(), **_tol(dtype))
+    wide = (4 * torch.randn(33, 2 * 64, generator=g, device=DEV)).to(dtype)          # rows in 16-byte pieces
+    wide[0, :8] = torch.tensor([-30.0, -9.0, -1.0, -1e-3, 0.0, 1e-3, 9.0, 30.0], device=DEV).to(dtype)
+    torch.testing.assert_close(activation.GeluTanhAndMul()(wide).float(), ref.GeluTanhAndMul()(wide).float(), **_tol(dtype))
 
 
 def _attention_pair(H, G, D, Dv, **kw):
