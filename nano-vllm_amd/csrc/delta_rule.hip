@@ -16,7 +16,9 @@
 //                          Everything after the raw projections is fp32.
 //
 // Layout of the recurrence: one workgroup per (sequence, head).  A lane owns one value column and a quarter of the
-// key rows (rows r, r + 4, ... of its quad index r), so the state lives in registers, both read-outs of a token
+// key rows (a contiguous run: its quad index r owns rows r * RPL .. r * RPL + RPL - 1, read from LDS four at a time; the
+// four runs sit RPL + 4 words apart so that the quad's 16-byte reads fall on different banks), so the state lives in
+// registers, both read-outs of a token
 // (S^T k and S^T q) are one pass over them and a two-step quad reduction, and the token loop has no workgroup
 // barrier: k, q, g, beta, v of 16 tokens are prepared into LDS by all waves together, each wave then runs the 16
 // tokens for its 16 columns, and the normalised read-out of the tile is written by all waves together.
@@ -59,6 +61,98 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
         acc += w[(int64_t)c * taps + (taps - 1 - j)] * xv;
     }
     y[(int64_t)t * y_stride + c] = (T)silu_f(acc);
+}
+
+// The same in 16-byte pieces: a thread takes 8 (bf16) or 4 (fp32) neighbouring channels of one token.
+template <typename T> struct Piece;
+template <> struct Piece<__bf16> {
+    static constexpr int n = 8;
+    static __device__ __forceinline__ void load(const __bf16* p, float* o) {
+        const uint4 u = *(const uint4*)p;
+        o[0] = bf16_lo(u.x); o[1] = bf16_hi(u.x); o[2] = bf16_lo(u.y); o[3] = bf16_hi(u.y);
+        o[4] = bf16_lo(u.z); o[5] = bf16_hi(u.z); o[6] = bf16_lo(u.w); o[7] = bf16_hi(u.w);
+    }
+    static __device__ __forceinline__ void store(__bf16* p, const float* o) {
+        *(uint4*)p = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+    }
+};
+template <> struct Piece<float> {
+    static constexpr int n = 4;
+    static __device__ __forceinline__ void load(const float* p, float* o) {
+        const float4 u = *(const float4*)p;
+        o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float* o) { *(float4*)p = make_float4(o[0], o[1], o[2], o[3]); }
+};
+
+
+// A thread keeps its channels' weights and the last `taps` inputs in registers and walks a run of tokens (16 in a large step, fewer when the step has too few rows to fill the chip that way): inside a
+// sequence every token costs one new 16-byte load; at a sequence's first row of the step the window is filled from
+// the carried state (or zeros before position 0).
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_silu_pieces_kernel(
+    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, const T* __restrict__ conv_state,
+    T* __restrict__ y, int64_t y_stride, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
+    const int* __restrict__ state_slots, int B, int C, int taps, int T_rows, int tokens_per_group) {
+    constexpr int N = Piece<T>::n;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * N;
+    if (c >= C) return;
+    float wt[kConvMaxTaps][N], win[kConvMaxTaps][N];        // wt[j], win[j]: weight of / input at the token j back
+#pragma unroll
+    for (int j = 0; j < kConvMaxTaps; ++j) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            wt[j][e] = j < taps ? w[(int64_t)(c + e) * taps + (taps - 1 - j)] : 0.f;
+            win[j][e] = 0.f;
+        }
+    }
+    const int t0 = blockIdx.x * tokens_per_group, t1 = min(T_rows, t0 + tokens_per_group);
+    int b = 0;
+    {
+        int lo = 0, hi = B;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (cu_q[mid] <= t0) lo = mid; else hi = mid;
+        }
+        b = lo;
+    }
+    for (int t = t0; t < t1; ++t) {
+        while (b + 1 < B && t >= cu_q[b + 1]) ++b;           // sequences without rows in this step are skipped
+        const int i = t - cu_q[b];
+        if (i == 0 || t == t0) {                             // fill the window's older entries
+            const int start = (cu_k[b + 1] - cu_k[b]) - (cu_q[b + 1] - cu_q[b]);
+            const T* st = conv_state + (int64_t)state_slots[b] * (taps - 1) * C;
+#pragma unroll
+            for (int j = 1; j < kConvMaxTaps; ++j) {
+                if (j < taps) {
+                    const int src = i - j;
+                    if (src >= 0) Piece<T>::load(x + (int64_t)(t - j) * x_stride + c, win[j]);
+                    else if (start + src >= 0) Piece<T>::load(st + (int64_t)(taps - 1 + src) * C + c, win[j]);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < N; ++e) win[j][e] = 0.f;
+                    }
+                }
+            }
+        }
+        Piece<T>::load(x + (int64_t)t * x_stride + c, win[0]);
+        float acc[N];
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < kConvMaxTaps; ++j) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) acc[e] += wt[j][e] * win[j][e];       // wt[j] = 0 for j >= taps
+        }
+#pragma unroll
+        for (int e = 0; e < N; ++e) acc[e] = silu_f(acc[e]);
+        Piece<T>::store(y + (int64_t)t * y_stride + c, acc);
+#pragma unroll
+        for (int j = kConvMaxTaps - 1; j > 0; --j) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) win[j][e] = win[j - 1][e];
+        }
+    }
 }
 
 template <typename T>
@@ -108,7 +202,7 @@ __global__ void gated_delta_rule_kernel(
     const float* __restrict__ dt_bias, const float* __restrict__ norm_w, float* __restrict__ state,
     T* __restrict__ out, int64_t out_stride, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ state_slots, int H, int G, int D, int Dv, float eps, int kDrTile) {
-    constexpr int DP = RPL * 4;                       // padded key rows
+    constexpr int DP = (RPL + 4) * 4;                 // LDS words per token and vector: four runs of RPL rows, padded
     extern __shared__ float smem[];
     float* ks = smem;                                 // [tile][DP]
     float* qs = ks + kDrTile * DP;                    // [tile][DP]
@@ -128,7 +222,7 @@ __global__ void gated_delta_rule_kernel(
     float S[RPL];
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
-        const int row = i * 4 + r;
+        const int row = r * RPL + i;
         S[i] = (live && start > 0 && row < D) ? S_slot[(int64_t)row * Dv + col] : 0.f;
     }
     const float rate = expf(A_log[h]);
@@ -151,7 +245,8 @@ __global__ void gated_delta_rule_kernel(
             qq = wave_sum(qq);
             const float kn = 1.0f / sqrtf(kk + 1e-6f), qn = q_scale / sqrtf(qq + 1e-6f);
             float kq = 0.f;
-            for (int d = lane; d < DP; d += 64) {
+            for (int d = lane; d < 4 * RPL; d += 64) {
+                const int at = tt * DP + (d / RPL) * (RPL + 4) + (d % RPL);
                 float kv = 0.f, qv = 0.f, gv = 1.f;
                 if (d < D) {
                     kv = (float)kr[d] * kn;
@@ -159,9 +254,9 @@ __global__ void gated_delta_rule_kernel(
                     const float a = (float)a_raw[t * a_stride + (int64_t)h * D + d] + dt_bias[(int64_t)h * D + d];
                     gv = expf(-rate * softplus_f(a));
                 }
-                ks[tt * DP + d] = kv;
-                qs[tt * DP + d] = qv;
-                gs[tt * DP + d] = gv;
+                ks[at] = kv;
+                qs[at] = qv;
+                gs[at] = gv;
                 kq += kv * qv;
             }
             kq = wave_sum(kq);
@@ -175,22 +270,26 @@ __global__ void gated_delta_rule_kernel(
         // ---- the recurrence over the tile, no barrier inside ---------------------------------------------
         if (live) {
             for (int tt = 0; tt < nt; ++tt) {
-                const float* kt = ks + tt * DP;
-                const float* qt = qs + tt * DP;
-                const float* gt = gs + tt * DP;
+                const float4* kt = (const float4*)(ks + tt * DP + r * (RPL + 4));
+                const float4* qt = (const float4*)(qs + tt * DP + r * (RPL + 4));
+                const float4* gt = (const float4*)(gs + tt * DP + r * (RPL + 4));
                 float sk = 0.f, sq = 0.f;
+                float4 kk[RPL / 4];
 #pragma unroll
-                for (int i = 0; i < RPL; ++i) {
-                    const int row = i * 4 + r;
-                    S[i] *= gt[row];
-                    sk += S[i] * kt[row];
-                    sq += S[i] * qt[row];
+                for (int i = 0; i < RPL / 4; ++i) {
+                    const float4 g4 = gt[i], q4 = qt[i];
+                    kk[i] = kt[i];
+                    S[4 * i] *= g4.x; S[4 * i + 1] *= g4.y; S[4 * i + 2] *= g4.z; S[4 * i + 3] *= g4.w;
+                    sk += S[4 * i] * kk[i].x + S[4 * i + 1] * kk[i].y + S[4 * i + 2] * kk[i].z + S[4 * i + 3] * kk[i].w;
+                    sq += S[4 * i] * q4.x + S[4 * i + 1] * q4.y + S[4 * i + 2] * q4.z + S[4 * i + 3] * q4.w;
                 }
                 sk = quad_sum(sk);
                 sq = quad_sum(sq);
                 const float u = bs[tt] * (vs[tt * Dv + col] - sk);
 #pragma unroll
-                for (int i = 0; i < RPL; ++i) S[i] += kt[i * 4 + r] * u;
+                for (int i = 0; i < RPL / 4; ++i) {
+                    S[4 * i] += kk[i].x * u; S[4 * i + 1] += kk[i].y * u; S[4 * i + 2] += kk[i].z * u; S[4 * i + 3] += kk[i].w * u;
+                }
                 if (r == 0) os[tt * Dv + col] = sq + u * bs[kDrTile + tt];     // (S + k u^T)^T q
             }
         }
@@ -211,7 +310,7 @@ __global__ void gated_delta_rule_kernel(
     if (live) {
 #pragma unroll
         for (int i = 0; i < RPL; ++i) {
-            const int row = i * 4 + r;
+            const int row = r * RPL + i;
             if (row < D) S_slot[(int64_t)row * Dv + col] = S[i];
         }
     }
@@ -227,7 +326,7 @@ static int launch_delta(const void* q, const void* k, const void* v, int64_t q_s
     const int waves = (Dv + 15) / 16;
     const dim3 grid((unsigned)B, (unsigned)H), block((unsigned)waves * 64);
     const int rpl = D <= 32 ? 8 : D <= 64 ? 16 : D <= 128 ? 32 : 64;
-    const size_t per_token = sizeof(float) * (size_t)(3 * rpl * 4 + 2 * Dv + 2);
+    const size_t per_token = sizeof(float) * (size_t)(3 * (rpl + 4) * 4 + 2 * Dv + 2);
     const int tile = (int)std::max<size_t>(1, std::min<size_t>(kDrMaxTile, kDrLdsBudget / per_token));
     const size_t smem = per_token * tile;
 #define NV_DR_CASE(R)                                                                                              \
@@ -264,7 +363,17 @@ extern "C" int nv_causal_conv_silu(const void* x, int64_t x_stride, const float*
     NV_REQUIRE(T < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_causal_conv_silu: launch too large");
     hipStream_t s = (hipStream_t)stream;
     const unsigned cb = (unsigned)((C + 255) / 256);
+    const int n = dtype == NV_DTYPE_BF16 ? 8 : 4;              // channels in a 16-byte piece
+    const bool pieces = C % n == 0 && x_stride % n == 0 && y_stride % n == 0 &&
+                        ((uintptr_t)x | (uintptr_t)y | (uintptr_t)conv_state) % 16 == 0;
+    const unsigned pb = (unsigned)((C / n + 255) / 256);
+    const int tpg = T * pb >= 8192 ? 16 : T * pb >= 2048 ? 4 : 1;      // tokens per workgroup: at least 512 workgroups
     if (dtype == NV_DTYPE_BF16) {
+        if (pieces)
+            hipLaunchKernelGGL(causal_conv_silu_pieces_kernel<__bf16>, dim3((unsigned)((T + tpg - 1) / tpg), pb), dim3(256), 0, s,
+                               (const __bf16*)x, x_stride, w, (const __bf16*)conv_state, (__bf16*)y, y_stride,
+                               cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg);
+        else
         hipLaunchKernelGGL(causal_conv_silu_kernel<__bf16>, dim3((unsigned)T, cb), dim3(256), 0, s, (const __bf16*)x,
                            x_stride, w, (const __bf16*)conv_state, (__bf16*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
                            state_slots, num_seqs, C, taps);
@@ -273,6 +382,11 @@ extern "C" int nv_causal_conv_silu(const void* x, int64_t x_stride, const float*
                                (const __bf16*)x, x_stride, (__bf16*)conv_state, cu_seqlens_q, cu_seqlens_k,
                                state_slots, C, taps);
     } else {
+        if (pieces)
+            hipLaunchKernelGGL(causal_conv_silu_pieces_kernel<float>, dim3((unsigned)((T + tpg - 1) / tpg), pb), dim3(256), 0, s,
+                               (const float*)x, x_stride, w, (const float*)conv_state, (float*)y, y_stride,
+                               cu_seqlens_q, cu_seqlens_k, state_slots, num_seqs, C, taps, (int)T, tpg);
+        else
         hipLaunchKernelGGL(causal_conv_silu_kernel<float>, dim3((unsigned)T, cb), dim3(256), 0, s, (const float*)x,
                            x_stride, w, (const float*)conv_state, (float*)y, y_stride, cu_seqlens_q, cu_seqlens_k,
                            state_slots, num_seqs, C, taps);

@@ -194,8 +194,9 @@ def test_scoremod_attention_single_rows_key_slices_and_head_groups(dtype, shape,
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 3, 4])
-def test_short_conv_in_portions_matches_one_pass(dtype, taps):
-    C, slots_n = 200, 5
+@pytest.mark.parametrize("C", [200, 203])          # rows in 16-byte pieces, and a width that has none
+def test_short_conv_in_portions_matches_one_pass(dtype, taps, C):
+    slots_n = 5
     a, r = delta_rule.ShortConvSilu(C, taps, device=DEV), ref.ShortConvSilu(C, taps, device=DEV)
     g = torch.Generator(device=DEV).manual_seed(taps)
     with torch.no_grad():
