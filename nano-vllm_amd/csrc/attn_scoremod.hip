@@ -372,7 +372,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     float* __restrict__ ws, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int D, int Dv, int block_size, float scale,
     float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2) {
+    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per round, min(kDecRep, H / G): sizes the LDS arrays
     extern __shared__ float dsm[];
     const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
     const int t = cu_q[b];
@@ -382,10 +382,10 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int VN = Vec16<T>::n;
     const int rs = 2 + Dv;
-    float* qs = dsm;                                          // [kDecRep][D]
-    float* ps = qs + kDecRep * D;                             // [4 waves][kDecRep][64]
-    float* red = ps + 4 * kDecRep * 64;                       // [4 waves][kDecRep][2 + Dv]
-    int64_t* rws = (int64_t*)(red + 4 * kDecRep * rs + ((4 * kDecRep * rs + kDecRep * D) & 1));   // [4 waves][64] rows
+    float* qs = dsm;                                          // [repm][D]
+    float* ps = qs + repm * D;                                // [4 waves][repm][64]
+    float* red = ps + 4 * repm * 64;                          // [4 waves][repm][2 + Dv]
+    int64_t* rws = (int64_t*)(red + 4 * repm * rs + ((4 * repm * rs + repm * D) & 1));   // [4 waves][64] rows
     const int* table = block_tables + (int64_t)b * max_blocks;
     const int k_lo = split * slice_keys, k_hi = min(n_keys, k_lo + slice_keys);
     // value pass: a V row is cut into 16-byte pieces; lane (sub, piece) = (lane >> cpr_log2, lane & (2^cpr_log2 - 1))
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
 #pragma unroll
             for (int i = 0; i < VN; ++i) acc[r][i] = 0.f;
         }
-        float* pw = ps + (wave * kDecRep) * 64;
+        float* pw = ps + (wave * repm) * 64;
         int64_t* rw = rws + wave * 64;
         // the slice's 64-key tiles go round the four waves
         for (int base = k_lo + wave * 64; base < k_hi; base += 4 * 64) {
@@ -484,7 +484,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
 #pragma unroll
                     for (int e = 0; e < VN; ++e) acc[r][e] += __shfl_xor(acc[r][e], o);
                 }
-                float* dst = red + ((wave * kDecRep) + r) * rs;
+                float* dst = red + ((wave * repm) + r) * rs;
                 if (lane == 0) {
                     dst[0] = m[r];
                     dst[1] = l[r];
@@ -499,13 +499,13 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
         for (int r = wave; r < rep; r += 4) {                 // wave w finishes heads w, w + 4, ...
             float mm = -INFINITY;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) mm = fmaxf(mm, red[(w * kDecRep + r) * rs]);
+            for (int w = 0; w < 4; ++w) mm = fmaxf(mm, red[(w * repm + r) * rs]);
             float ll = 0.f, f[4];
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const float mw = red[(w * kDecRep + r) * rs];
+                const float mw = red[(w * repm + r) * rs];
                 f[w] = mw == -INFINITY ? 0.f : expf(mw - mm);  // a wave (or the whole slice) may have had no keys
-                ll += f[w] * red[(w * kDecRep + r) * rs + 1];
+                ll += f[w] * red[(w * repm + r) * rs + 1];
             }
             const int head = head0 + r;
             if (splits == 1) {
@@ -518,7 +518,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                 for (int c = lane; c < Dv; c += 64) {
                     float o = 0.f;
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) o += f[w] * red[(w * kDecRep + r) * rs + 2 + c];
+                    for (int w = 0; w < 4; ++w) o += f[w] * red[(w * repm + r) * rs + 2 + c];
                     out[(int64_t)t * out_stride + (int64_t)head * Dv + c] = (T)(o * osc / den);
                 }
             } else {
@@ -530,7 +530,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                 for (int c = lane; c < Dv; c += 64) {
                     float o = 0.f;
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) o += f[w] * red[(w * kDecRep + r) * rs + 2 + c];
+                    for (int w = 0; w < 4; ++w) o += f[w] * red[(w * repm + r) * rs + 2 + c];
                     wrow[2 + c] = o;
                 }
             }
@@ -654,7 +654,8 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     // Sequences with one row: the decode kernel (key slices, the query heads of a group together) when rows can be
     // read in 16-byte pieces, else the row-per-wave kernel.
     const int vn = bf ? 8 : 4;
-    const size_t dec_lds = sizeof(float) * ((size_t)kDecRep * D + 4 * kDecRep * 64 + 4 * kDecRep * (2 + Dv) + 1) +
+    const int repm = std::min(kDecRep, H / G);
+    const size_t dec_lds = sizeof(float) * ((size_t)repm * D + 4 * repm * 64 + 4 * repm * (2 + Dv) + 1) +
                            sizeof(int64_t) * 4 * 64;
     int cpr_log2 = 0;                                          // 16-byte pieces per V row, rounded up to a power of two
     while ((vn << cpr_log2) < Dv) ++cpr_log2;
@@ -688,7 +689,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
 #define NV_DEC_ARGS(TT)                                                                                              \
     (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, (TT*)out, (float*)workspace, cu_seqlens_q, cu_seqlens_k, \
         block_tables, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,        \
-        q_stride, out_stride, plan.splits, plan.slice_keys, T, cpr_log2
+        q_stride, out_stride, plan.splits, plan.slice_keys, T, cpr_log2, repm
         if (bf) hipLaunchKernelGGL(attn_scoremod_decode_kernel<__bf16>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(__bf16));
         else hipLaunchKernelGGL(attn_scoremod_decode_kernel<float>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(float));
 #undef NV_DEC_ARGS
