@@ -4,8 +4,8 @@
 //   s_ij = cap * tanh(s_ij / cap)                  if cap > 0            (logit soft-capping)
 //   s_ij = s_ij + bias[h][min(i - j, n_dist-1)]    if bias given         (learned distance bias, one row per head;
 //                                                                         the host expands bucketed tables)
-//   p_ij = exp(s_ij) / (sum_j' exp(s_ij') + exp(sink_h))                 (sink: an extra term of the denominator
-//                                                                         with no key and no value, if given)
+//   p_ij = exp(s_ij) / (sum_j' exp(s_ij') + exp(sink_h))                 (sink: a learned per-head logit that joins
+//                                                                         the normalisation only, if given)
 //
 // Causal (key position <= query position), grouped heads (query head h reads kv head h / (H / G)), any head size:
 // the key size D and the value size Dv are runtime arguments and may differ.  K/V are read through the block table
@@ -346,7 +346,7 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
 // keeping one piece of every head's accumulator.  No barrier inside the loop.  The
 // waves' running (max, sum, accumulator) are joined through LDS, and the slices through a workspace and a second
 // small launch that also puts the sink into the denominator.
-constexpr int kDecRep = 8;             // query heads per kv head handled at once (larger groups go round again)
+constexpr int kDecRep = 8;             // query heads per kv head handled at once (larger groups take further passes)
 constexpr int kDecThreads = 256;
 
 template <typename T> struct Vec16;
@@ -372,7 +372,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     float* __restrict__ ws, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int D, int Dv, int block_size, float scale,
     float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per round, min(kDecRep, H / G): sizes the LDS arrays
+    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per pass, min(kDecRep, H / G): sizes the LDS arrays
     extern __shared__ float dsm[];
     const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
     const int t = cu_q[b];
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
         }
         float* pw = ps + (wave * repm) * 64;
         int64_t* rw = rws + wave * 64;
-        // the slice's 64-key tiles go round the four waves
+        // the slice's 64-key tiles are dealt to the four waves in turn
         for (int base = k_lo + wave * 64; base < k_hi; base += 4 * 64) {
             const int j = base + lane;
             const bool live = j < k_hi;

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------ delta rule
-constexpr int kDrMaxTile = 16;     // tokens prepared per round, fewer when LDS is short
+constexpr int kDrMaxTile = 16;     // tokens prepared at a time, fewer when LDS is short
 constexpr int kDrLdsBudget = 60 * 1024;
 
 template <int CTRL>

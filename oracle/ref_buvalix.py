@@ -110,8 +110,11 @@ def short_conv_silu(x, w, dtype=torch.float32):
 
 
 def gated_delta_channel(q, k, v, beta, g):
-    """Per head, token by token: S <- g * S (rows = key channels); u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
-    q, k: [T, H, D]; v: [T, H, Dv]; beta: [T, H]; g: [T, H, D].  fp32 state, zero at the start."""
+    """The recurrence of one head, written as three assignments per token t (S_t is [D, Dv], rows indexed by key channel):
+        A   = Diag(g_t) S_{t-1}                 decay
+        S_t = A + k_t (beta_t (v_t - A^T k_t))^T  delta-rule write
+        o_t = S_t^T q_t                          read after the write
+    q, k: [T, H, D]; v: [T, H, Dv]; beta: [T, H]; g: [T, H, D].  S_0 = 0, float32 throughout."""
     T, H, D = q.shape
     Dv = v.shape[-1]
     S = torch.zeros(H, D, Dv)

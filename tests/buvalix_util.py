@@ -16,7 +16,7 @@ def attention_layer(heads=4, kv_heads=2, dim=24, vdim=40, rot_dims=12, base=500.
                       "softcap": softcap, "rot": {"dims": rot_dims, "base": base}}}
 
 
-def attention2_layer(heads=6, kv_heads=3, dim=16, vdim=8, coef=0.5, every=7, bias_max=40, softcap=30.0, ff=32):
+def attention2_layer(heads=6, kv_heads=3, dim=16, vdim=8, coef=0.4, every=7, bias_max=40, softcap=30.0, ff=32):
     return {"type": "attention_2", "mlp": None if ff is None else {"kind": "dense", "ff": ff},
             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": 1.3 * dim ** -0.5,
                       "softcap": softcap, "q_temp": {"coef": coef, "every": every}, "bias_max": bias_max}}

@@ -103,7 +103,7 @@ def kernel_records(dev):
         T = sum(n_qs)
         q, k, v = rn(T, H, D), rn(T, G, D), rn(T, G, D)
         kc, vc = rn(nb, bs, G, D), rn(nb, bs, G, D)
-        attn = attention.ScoreModAttention(H, G, D, D, scale, softcap=50.0, rot_dims=64, rot_base=1e4, use_sink=True, device=dev)
+        attn = attention.ScoreModAttention(H, G, D, D, scale, softcap=30.0, rot_dims=64, rot_base=1e4, use_sink=True, device=dev)
         nv.set_context(ctx)
         pairs = sum(nq * (nk - nq) + nq * (nq + 1) // 2 for nq, nk in zip(n_qs, n_ks))
         flops = 4 * D * H * pairs
@@ -117,7 +117,7 @@ def kernel_records(dev):
         rec["like: qknorm_rope_store"] = rate(t, nbytes=T * (2 * H + 4 * G) * D * 2)
         singles = int(max(n_qs) == 1)
         t = timed(lambda: ops.attn_scoremod_paged(q, kc, vc, ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.block_tables, scale,
-                                                  50.0, attn.sink, None, max(n_qs), max(n_ks), singles))
+                                                  30.0, attn.sink, None, max(n_qs), max(n_ks), singles))
         if singles:
             rec["attn_scoremod (single rows)"] = rate(t, nbytes=kv_bytes)
             t = timed(lambda: ops.attn_decode_paged(q, kc, vc, ctx.cu_seqlens_k, ctx.block_tables, max(n_ks), scale))
@@ -158,7 +158,7 @@ def kernel_records(dev):
 
 
 def buvalix_config(width, ff, n_groups, vocab):
-    att = {"heads": 16, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0}
+    att = {"heads": 16, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0}
     group = [
         {"type": "channel_delta", "mlp": {"kind": "dense", "ff": ff},
          "mixer": {"heads": 16, "kv_heads": 16, "dim": 128, "vdim": 128, "conv": 4}},
@@ -172,7 +172,7 @@ def buvalix_config(width, ff, n_groups, vocab):
             "loop": {"start": 0, "stop": 0, "times": 1}}
 
 
-def random_buvalix(cfg_dict, dev, dtype, rank=64, rel_rows=32):
+def random_buvalix(cfg_dict, dev, dtype, rank=64, rel_rows=24):
     cfg = BuvalixConfig.from_dict(cfg_dict)
     model = BuvalixForCausalLM(cfg, dtype=dtype, device=dev)
     g = torch.Generator().manual_seed(0)
