@@ -366,13 +366,15 @@ __device__ __forceinline__ void load16<float>(const float* p, float* o) {
     const float4 u = *(const float4*)p;
     o[0] = u.x; o[1] = u.y; o[2] = u.z; o[3] = u.w;
 }
-template <typename T>
+// REP: query heads of a group taken per pass (1, 2, 4 or 8): the per-head registers are sized by it, so small groups
+// run at high occupancy.
+template <typename T, int REP>
 __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     float* __restrict__ ws, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int D, int Dv, int block_size, float scale,
     float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per pass, min(kDecRep, H / G): sizes the LDS arrays
+    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per pass (= REP): sizes the LDS arrays
     extern __shared__ float dsm[];
     const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
     const int t = cu_q[b];
@@ -392,16 +394,16 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     // takes piece `piece` of every (64 >> cpr_log2)-th key, so one load instruction of the wave covers several whole rows
     const int piece = lane & ((1 << cpr_log2) - 1), sub = lane >> cpr_log2, rows_per_load = 64 >> cpr_log2;
     const bool piece_live = piece * VN < Dv;
-    for (int h0 = 0; h0 < rep_all; h0 += kDecRep) {
-        const int rep = min(kDecRep, rep_all - h0);
+    for (int h0 = 0; h0 < rep_all; h0 += REP) {
+        const int rep = min(REP, rep_all - h0);
         const int head0 = g * rep_all + h0;
         __syncthreads();
         for (int i = tid; i < rep * D; i += kDecThreads)
             qs[i] = (float)q[(int64_t)t * q_stride + (int64_t)(head0 + i / D) * D + (i % D)];
         __syncthreads();
-        float m[kDecRep], l[kDecRep], acc[kDecRep][VN];
+        float m[REP], l[REP], acc[REP][VN];
 #pragma unroll
-        for (int r = 0; r < kDecRep; ++r) {
+        for (int r = 0; r < REP; ++r) {
             m[r] = -INFINITY;
             l[r] = 0.f;
 #pragma unroll
@@ -413,9 +415,9 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
         for (int base = k_lo + wave * 64; base < k_hi; base += 4 * 64) {
             const int j = base + lane;
             const bool live = j < k_hi;
-            float sc[kDecRep];
+            float sc[REP];
 #pragma unroll
-            for (int r = 0; r < kDecRep; ++r) sc[r] = 0.f;
+            for (int r = 0; r < REP; ++r) sc[r] = 0.f;
             int64_t row = 0;
             if (live) {
                 row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
@@ -425,7 +427,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                     float kv[VN];
                     load16<T>(kr + d, kv);
 #pragma unroll
-                    for (int r = 0; r < kDecRep; ++r) {
+                    for (int r = 0; r < REP; ++r) {
                         if (r < rep) {
 #pragma unroll
                             for (int e = 0; e < VN; ++e) sc[r] += qs[r * D + d + e] * kv[e];
@@ -434,9 +436,9 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                 }
             }
             rw[lane] = row;
-            float corr[kDecRep];
+            float corr[REP];
 #pragma unroll
-            for (int r = 0; r < kDecRep; ++r) {
+            for (int r = 0; r < REP; ++r) {
                 corr[r] = 1.f;
                 if (r < rep) {
                     float x = -INFINITY;
@@ -466,7 +468,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                     float vv[VN];
                     load16<T>(v_cache + rw[jj] * Dv + piece * VN, vv);
 #pragma unroll
-                    for (int r = 0; r < kDecRep; ++r) {
+                    for (int r = 0; r < REP; ++r) {
                         if (r < rep) {
                             const float pj = pw[r * 64 + jj];
 #pragma unroll
@@ -478,7 +480,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
         }
         // ---- join the lanes that share a piece, then the four waves ---------------------------------------------
 #pragma unroll
-        for (int r = 0; r < kDecRep; ++r) {
+        for (int r = 0; r < REP; ++r) {
             if (r < rep) {
                 for (int o = 1 << cpr_log2; o < 64; o <<= 1) {
 #pragma unroll
@@ -654,7 +656,8 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     // Sequences with one row: the decode kernel (key slices, the query heads of a group together) when rows can be
     // read in 16-byte pieces, else the row-per-wave kernel.
     const int vn = bf ? 8 : 4;
-    const int repm = std::min(kDecRep, H / G);
+    const int rep_group = std::min(kDecRep, H / G);
+    const int repm = rep_group <= 2 ? rep_group : rep_group <= 4 ? 4 : 8;       // heads per pass: the kernel's REP
     const size_t dec_lds = sizeof(float) * ((size_t)repm * D + 4 * repm * 64 + 4 * repm * (2 + Dv) + 1) +
                            sizeof(int64_t) * 4 * 64;
     int cpr_log2 = 0;                                          // 16-byte pieces per V row, rounded up to a power of two
@@ -690,8 +693,16 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, (TT*)out, (float*)workspace, cu_seqlens_q, cu_seqlens_k, \
         block_tables, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,        \
         q_stride, out_stride, plan.splits, plan.slice_keys, T, cpr_log2, repm
-        if (bf) hipLaunchKernelGGL(attn_scoremod_decode_kernel<__bf16>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(__bf16));
-        else hipLaunchKernelGGL(attn_scoremod_decode_kernel<float>, dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(float));
+#define NV_DEC_LAUNCH(TT, R) \
+    hipLaunchKernelGGL((attn_scoremod_decode_kernel<TT, R>), dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(TT))
+#define NV_DEC_BY_REP(TT)                     \
+    if (repm == 1) NV_DEC_LAUNCH(TT, 1);      \
+    else if (repm == 2) NV_DEC_LAUNCH(TT, 2); \
+    else if (repm <= 4) NV_DEC_LAUNCH(TT, 4); \
+    else NV_DEC_LAUNCH(TT, 8);
+        if (bf) { NV_DEC_BY_REP(__bf16) } else { NV_DEC_BY_REP(float) }
+#undef NV_DEC_BY_REP
+#undef NV_DEC_LAUNCH
 #undef NV_DEC_ARGS
         int rc = check_launch("nv_attn_scoremod_paged (decode kernel)");
         if (rc != NV_OK) return rc;
