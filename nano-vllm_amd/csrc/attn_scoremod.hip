@@ -182,8 +182,9 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
 constexpr int kTileQ = 64, kTileK = 64, kTileThreads = 256;
 
 __device__ __forceinline__ float fast_tanh(float x) {
-    // 1 - 2 / (e^{2x} + 1): exact limits at both ends (e^{2x} -> inf gives 1, -> 0 gives -1)
-    return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f);
+    // 1 - 2 / (e^{2x} + 1) with the hardware exponential and reciprocal (about 1 ulp each; the result feeds a bf16
+    // probability): exact limits at both ends (e^{2x} -> inf gives 1, -> 0 gives -1)
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * 2.885390081777927f) + 1.0f);
 }
 
 template <int DS, int DVS>     // D = 16 DS, Dv = 16 DVS: every loop below has a compile-time length
@@ -198,9 +199,11 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
     const int q0 = cu_q[b], len_q = cu_q[b + 1] - q0, len_k = cu_k[b + 1] - cu_k[b];
     if (len_q <= 1 || qt * kTileQ >= len_q) return;          // single rows belong to the row-wave kernel
     const int g = h / (H / G);
-    const int k_ld = D + 8, v_ld = kTileK + 8;                // LDS row lengths in elements (16-byte multiples)
-    __bf16* ldsK = (__bf16*)lds_raw;                          // [64][D + 8]
-    __bf16* ldsV = ldsK + kTileK * k_ld;                      // [Dv][64 + 8]
+    // LDS row lengths in elements: 2 words more than a multiple of 32 words, so the 16 lanes that read 8 bytes of 16
+    // different rows in one pass of an operand load fall on 16 different bank pairs
+    const int k_ld = D + 4, v_ld = kTileK + 4;
+    __bf16* ldsK = (__bf16*)lds_raw;                          // [64][D + 4]
+    __bf16* ldsV = ldsK + kTileK * k_ld;                      // [Dv][64 + 4]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 15, lg = lane >> 4;
     const int start = len_k - len_q;                          // position of the sequence's first row in this step
@@ -245,7 +248,11 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
     for (int base = 0; base <= last_pos; base += kTileK) {
         __syncthreads();                                      // the previous tile has been consumed
 #pragma unroll
-        for (int i = 0; i < KP; ++i) *(uint4*)(ldsK + my_key * k_ld + 8 * (my_quarter + 4 * i)) = kreg[i];
+        for (int i = 0; i < KP; ++i) {                        // rows are 8-byte aligned: two 8-byte stores
+            uint2* dst = (uint2*)(ldsK + my_key * k_ld + 8 * (my_quarter + 4 * i));
+            dst[0] = make_uint2(kreg[i].x, kreg[i].y);
+            dst[1] = make_uint2(kreg[i].z, kreg[i].w);
+        }
 #pragma unroll
         for (int i = 0; i < VP; ++i) {
             // V goes in transposed; consecutive lanes hold consecutive keys, so each of the eight 2-byte stores of a
@@ -649,7 +656,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     const bool bf = dtype == NV_DTYPE_BF16;
     const bool several = max_seqlen_q != 1, singles = single_rows != 0;      // what the step may hold
     // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes 32, 64, 96 or 128, aligned rows), else the row-per-wave kernel.
-    const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 8) + (size_t)Dv * (kTileK + 8));
+    const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 4) + (size_t)Dv * (kTileK + 4));
     const auto tile_size = [](int n) { return n == 32 || n == 64 || n == 96 || n == 128; };      // built tile shapes
     const bool tile_ok = bf && max_seqlen_q > 1 && tile_size(D) && tile_size(Dv) && tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
                          ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
