@@ -442,7 +442,9 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                     }
                 }
             }
-            rw[lane] = row;
+            // a lane past the slice names the tile's first key (always live): its weight is 0, and 0 times a row that was
+            // really written is 0, whatever unwritten cache memory holds
+            rw[lane] = live ? row : __shfl(row, 0);
             float corr[REP];
 #pragma unroll
             for (int r = 0; r < REP; ++r) {
@@ -467,8 +469,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
                     for (int i = 0; i < VN; ++i) acc[r][i] *= corr[r];
                 }
             }
-            // the tile's V rows (the wave reads its own LDS words: no workgroup barrier needed); keys past the slice
-            // have weight 0 and row 0, which is a row of the cache like any other
+            // the tile's V rows (the wave reads its own LDS words: no workgroup barrier needed)
             if (piece_live) {
 #pragma unroll 4
                 for (int jj = sub; jj < 64; jj += rows_per_load) {
