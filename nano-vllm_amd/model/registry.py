@@ -89,7 +89,18 @@ def _buvalix_model(cfg, dtype=torch.bfloat16, device="cuda", **kw):
     return BuvalixForCausalLM(cfg, dtype=dtype, device=device, **kw)
 
 
+def _benarax_config(raw: dict):
+    from .benarax import BenaraxConfig
+    return BenaraxConfig.from_dict(raw)
+
+
+def _benarax_model(cfg, dtype=torch.bfloat16, device="cuda", **kw):
+    from .benarax import BenaraxForCausalLM
+    return BenaraxForCausalLM(cfg, dtype=dtype, device=device, **kw)
+
+
 register(["Qwen3ForCausalLM", "Qwen3"], _qwen3_config, lambda cfg, **kw: _qwen3_model(cfg, **kw))
 register(["LlamaForCausalLM", "Llama"], lambda raw: _qwen3_config({**raw, "qk_norm": False}),
          lambda cfg, **kw: _qwen3_model(cfg, **kw))
 register(["Buvalix", "BuvalixForCausalLM"], _buvalix_config, _buvalix_model)
+register(["Benarax", "BenaraxForCausalLM"], _benarax_config, _benarax_model)
