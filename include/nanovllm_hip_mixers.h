@@ -104,6 +104,94 @@ NV_API int nv_gated_delta_rule(const void* q, const void* k, const void* v, int6
                                const int32_t* state_slots, int num_seqs, int H, int G, int D, int Dv, float eps,
                                int dtype, void* stream);
 
+/* -------------------------------------------------------------------------------------------------
+ * An fp32 stream with one grouped RMS norm per layer, parallel sublayers and a normalised side input.
+ * ------------------------------------------------------------------------------------------------- */
+/*
+ * One boundary of an fp32 residual stream, per row and in place (every part optional):
+ *   r <- r + mult * (add + sum_j parts[:, j])       add: [rows, cols] of dtype (row stride add_stride);
+ *                                                   parts: [rows, n_parts, cols] fp32 contiguous
+ *   r <- r + mult * n / sqrt(mean(n^2) + eps) * normed_w         normed: [rows, cols] of dtype
+ *   copy <- r (dtype, contiguous)
+ *   y32 / y <- grouped RMS norm of r times norm_w: the row is cut into `groups` equal consecutive parts and each is
+ *   divided by its own sqrt(mean(part^2) + eps); y32 fp32, y of dtype, either or both.
+ * cols <= 16384, groups <= 1024 and a divisor of cols.
+ */
+NV_API int nv_stream_boundary(void* resid, const void* add, int64_t add_stride, const void* parts, int n_parts,
+                              const void* normed, int64_t normed_stride, const float* normed_w, float mult,
+                              const float* norm_w, int groups, float eps, void* y32, void* y, void* copy, int dtype,
+                              int64_t rows, int cols, void* stream);
+
+/* y = x / sqrt(mean(x^2) + eps) * w per row; x (row stride x_stride) and y (contiguous) of dtype, w fp32. */
+NV_API int nv_rms_norm_rows(const void* x, int64_t x_stride, const float* w, void* y, int dtype, int64_t rows,
+                            int cols, float eps, void* stream);
+
+/*
+ * y[t, c] = x[t, c] + sum_j w[c, j] * x[t - taps + 1 + j, c]: a causal convolution over time per channel, added to its
+ * input.  x: [T, C] fp32 contiguous; w: [C, taps] fp32 (the last column multiplies the current token); y: [T, C] of
+ * y_dtype; conv_state: [num_slots, taps - 1, C] fp32, the last inputs of every sequence, updated.  A sequence at
+ * position 0 ignores what its slot holds.
+ */
+NV_API int nv_causal_conv_add(const float* x, const float* w, float* conv_state, void* y, int y_dtype,
+                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* state_slots,
+                              int num_seqs, int64_t T, int C, int taps, void* stream);
+
+/* y[t, j] = gelu_tanh(z[t, j]) * table[ids[t], offset + j], j < dim; z, table, y of dtype, y contiguous. */
+NV_API int nv_token_gate(const void* z, int64_t z_stride, const void* table, int64_t table_stride,
+                         const int64_t* ids, int offset, int dim, void* y, int dtype, int64_t T, void* stream);
+
+/*
+ * Generalized delta rule, state [num_slots, H, D, D] fp32 carried per slot (key channel x value channel):
+ *   u = k / sqrt(sum k^2 + key_eps);  w = exp(-decay_rate * sigmoid(w_raw + w_bias));  a = sigmoid(a_raw + a_bias)
+ *   S <- diag(w) S - (a * u)(u^T S) + k v^T        (both terms read the old state; token by token)
+ *   out[t, h] = (S^T r) / sqrt(mean((S^T r)^2) + eps) * norm_w[h] * sigmoid(gate_raw[t, h])
+ * r, k, v, w_raw, a_raw, gate_raw, out: [T, H, D] of dtype with token strides; w_bias, a_bias, norm_w: [H, D] fp32.
+ * D <= 256.
+ */
+NV_API int nv_general_delta_rule(const void* r, const void* k, const void* v, int64_t r_stride, int64_t k_stride,
+                                 int64_t v_stride, const void* w_raw, int64_t w_stride, const void* a_raw,
+                                 int64_t a_stride, const void* gate_raw, int64_t gate_stride, const float* w_bias,
+                                 const float* a_bias, const float* norm_w, float* state, void* out, int64_t out_stride,
+                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const int32_t* state_slots,
+                                 int num_seqs, int H, int D, float eps, float decay_rate, float key_eps, int dtype,
+                                 void* stream);
+
+/*
+ * In front of nv_attn_scoremod_paged when keys / values are cached as one normalised latent per token plus one rotated
+ * key part shared by all heads (attention in the latent space, G = 1, key size rank + R, value size rank):
+ *   c = ckv[t, :rank] / sqrt(mean(.^2) + eps) * latent_w;   k_r = rot(ckv[t, rank:])
+ *   q_full[t, h] = [q_lat[t, h] | rot(q[t, h, Dq - R:])];   k_cache[slot] = [c | k_r];   v_cache[slot] = c
+ * rot turns pair i by positions[t] * freq[i], cos and sin times mag; pairs (2i, 2i+1) if interleaved else (i, i + R/2).
+ * q: [T, H, Dq] (token stride q_stride); q_lat: [T, H, rank] with token / head strides; ckv: [T, rank + R];
+ * q_full: [T, H, rank + R] contiguous; k_cache: [num_slots, rank + R]; v_cache: [num_slots, rank].
+ */
+NV_API int nv_latent_prep_store(const void* q, int64_t q_stride, int Dq, const void* q_lat, int64_t ql_stride_t,
+                                int64_t ql_stride_h, const void* ckv, int64_t ckv_stride, const float* latent_w,
+                                const float* freq, float mag, int interleaved, const int64_t* positions,
+                                const int32_t* slot_mapping, void* q_full, void* k_cache, void* v_cache, int dtype,
+                                int64_t T, int H, int rank, int R, float eps, void* stream);
+
+/*
+ * Routed experts.  nv_moe_route: the `top` largest of every row of logits [T, E] (fp32), weights = softmax over the
+ * chosen; ids / weights: [T, top].  nv_moe_align: sorted_pairs [pairs] = the (token, choice) pairs ordered by expert,
+ * meta = [number of row tiles, then (expert, first position, rows) per tile], tiles of at most tile_rows (16 or 64,
+ * nv_moe_tile_rows suggests one) rows of one expert; meta holds 1 + 3 * nv_moe_max_tiles ints.  nv_moe_gate_up:
+ * y[position] = g * sigmoid(alpha g) * (u + 1), g = min(G_e h, limit), u = clamp(U_e h, -limit, limit), with
+ * gate_up: [E, 2 ff, width] (gate rows, then up rows), y: [pairs, ff] of dtype.  nv_moe_down: out[pair] =
+ * pair_weights[pair] * (D_e y[position]), down: [E, width, ff], out: [pairs, width] fp32.
+ */
+NV_API int nv_moe_route(const float* logits, int32_t* ids, float* weights, int64_t T, int E, int top, void* stream);
+NV_API int nv_moe_tile_rows(int64_t pairs, int E);
+NV_API int64_t nv_moe_max_tiles(int64_t pairs, int E, int tile_rows);
+NV_API int nv_moe_align(const int32_t* ids, int32_t* sorted_pairs, int32_t* meta, int64_t pairs, int E,
+                        int tile_rows, void* stream);
+NV_API int nv_moe_gate_up(const void* h, int64_t h_stride, const void* gate_up, const int32_t* sorted_pairs,
+                          const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width, int ff,
+                          float limit, float alpha, int tile_rows, void* stream);
+NV_API int nv_moe_down(const void* y, const void* down, const int32_t* sorted_pairs, const int32_t* meta,
+                       const float* pair_weights, float* out, int dtype, int64_t pairs, int E, int width, int ff,
+                       int tile_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,7 +12,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip.so")
 MIXERS_LIB_PATH = os.path.join(_HERE, "lib", "libnanovllm_hip_mixers.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -77,6 +77,21 @@ MIXERS_PROTOTYPES = {
     "nv_causal_conv_silu": (_i32, [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
     "nv_gated_delta_rule": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp,
                                    _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "nv_stream_boundary": (_i32, [_vp, _vp, _i64, _vp, _i32, _vp, _i64, _vp, _f32, _vp, _i32, _f32, _vp, _vp, _vp, _i32,
+                                  _i64, _i32, _vp]),
+    "nv_rms_norm_rows": (_i32, [_vp, _i64, _vp, _vp, _i32, _i64, _i32, _f32, _vp]),
+    "nv_causal_conv_add": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _vp]),
+    "nv_token_gate": (_i32, [_vp, _i64, _vp, _i64, _vp, _i32, _i32, _vp, _i32, _i64, _vp]),
+    "nv_general_delta_rule": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp,
+                                     _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _f32, _f32, _i32, _vp]),
+    "nv_latent_prep_store": (_i32, [_vp, _i64, _i32, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _f32, _i32, _vp, _vp, _vp, _vp,
+                                    _vp, _i32, _i64, _i32, _i32, _i32, _f32, _vp]),
+    "nv_moe_route": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "nv_moe_tile_rows": (_i32, [_i64, _i32]),
+    "nv_moe_max_tiles": (_i64, [_i64, _i32, _i32]),
+    "nv_moe_align": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "nv_moe_gate_up": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _i32, _vp]),
+    "nv_moe_down": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
 }
 DTYPE_BF16, DTYPE_F32 = 0, 1
 

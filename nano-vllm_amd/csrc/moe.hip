@@ -1,0 +1,275 @@
+// Routed experts (mixture of experts with small clamped-GLU experts), without a host round trip:
+//
+// nv_moe_route          per token, from fp32 router logits [T, E]: the `top` largest (lowest index first among equals),
+//                       their weights = softmax over the chosen logits only.  ids [T, top] int32, weights [T, top] fp32.
+// nv_moe_align          sorts the T * top (token, choice) pairs by expert: sorted_pairs[position] = pair index, and a
+//                       table of row tiles (expert, first position, rows) of at most `tile_rows` rows that never
+//                       straddle two experts, plus their count, all on the device.
+// nv_moe_gate_up        y[position, :] = act(G_e h, U_e h) for every sorted position (expert e, token of the pair):
+//                       g = min(G_e h, limit), u = clamp(U_e h, -limit, limit), act = g * sigmoid(alpha g) * (u + 1).
+// nv_moe_down           out[pair, :] = weight[pair] * (D_e y[position, :]), fp32, at the pair's own row: the caller sums
+//                       the `top` rows of a token in a fixed order (no atomics, bitwise reproducible).
+//
+// Both products are one grouped matrix product on the matrix cores: a workgroup of four waves takes one row tile
+// (16 or 64 rows of ONE expert) and 64 output columns, stages 32-deep slices of the rows and of the expert's weight
+// rows through LDS and issues v_mfma_f32_16x16x16_bf16 (bfloat16) or v_mfma_f32_16x16x4_f32 (true fp32) on them; a
+// wave owns 16 columns and all row sub-tiles, so every weight element is read from LDS once per 16 rows.  Weights are
+// [E, rows_out, rows_in] with the contraction index contiguous, as stored.  The launch is sized for the most tiles any
+// routing can produce; workgroups beyond the table's count return at once.
+#include <algorithm>
+
+#include "nv_common.h"
+#include "../../include/nanovllm_hip_mixers.h"
+
+namespace nv {
+
+constexpr int kMoeMaxTop = 16;
+constexpr int kMoeBN = 64, kMoeBK = 32;
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int* __restrict__ ids,
+                                                        float* __restrict__ wgt, int64_t T, int E, int top) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= T) return;
+    const float* z = logits + t * E;
+    int chosen[kMoeMaxTop];
+    float val[kMoeMaxTop];
+    for (int j = 0; j < top; ++j) {
+        int best = -1;
+        float bv = 0.f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
+            const float v = z[e];
+            if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
+        }
+        chosen[j] = best;
+        val[j] = bv;
+    }
+    float sum = 0.f;
+    const float top_logit = val[0];
+    for (int j = 0; j < top; ++j) {
+        val[j] = expf(val[j] - top_logit);
+        sum += val[j];
+    }
+    for (int j = 0; j < top; ++j) {
+        ids[t * top + j] = chosen[j];
+        wgt[t * top + j] = val[j] / sum;
+    }
+}
+
+// One workgroup.  meta: [0] = number of tiles, then (expert, first position, rows) per tile.
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, int* __restrict__ sorted_pairs,
+                                                         int* __restrict__ meta, int64_t P, int E, int tile_rows) {
+    extern __shared__ int sm[];                    // [E] counts, [E] cursors
+    int* count = sm;
+    int* cursor = sm + E;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += 1024) count[e] = 0;
+    __syncthreads();
+    for (int64_t p = tid; p < P; p += 1024) atomicAdd(&count[ids[p]], 1);
+    __syncthreads();
+    if (tid == 0) {
+        int off = 0, n = 0;
+        for (int e = 0; e < E; ++e) {
+            const int c = count[e];
+            cursor[e] = off;
+            for (int m = 0; m < c; m += tile_rows) {
+                meta[1 + 3 * n] = e;
+                meta[2 + 3 * n] = off + m;
+                meta[3 + 3 * n] = min(tile_rows, c - m);
+                ++n;
+            }
+            off += c;
+        }
+        meta[0] = n;
+    }
+    __syncthreads();
+    for (int64_t p = tid; p < P; p += 1024) sorted_pairs[atomicAdd(&cursor[ids[p]], 1)] = (int)p;
+}
+
+template <typename T> struct MoeMma;
+template <> struct MoeMma<__bf16> {
+    static constexpr int kVec = 8, kPad = 8, kStep = 16;
+    static __device__ __forceinline__ f32x4 run(const __bf16* a, const __bf16* b, int lg, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*(const s16x4*)(a + 4 * lg), *(const s16x4*)(b + 4 * lg), c, 0, 0, 0);
+    }
+};
+template <> struct MoeMma<float> {
+    static constexpr int kVec = 4, kPad = 4, kStep = 4;
+    static __device__ __forceinline__ f32x4 run(const float* a, const float* b, int lg, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a[lg], b[lg], c, 0, 0, 0);
+    }
+};
+
+// kVec elements of a row starting at k0 into LDS, zeros past K (or for a missing row)
+template <typename T>
+__device__ __forceinline__ void moe_stage(T* dst, const T* row, int k0, int K, bool vec_ok) {
+    constexpr int V = MoeMma<T>::kVec;
+    if (row != nullptr && vec_ok && k0 + V <= K) {
+        *(uint4*)dst = *(const uint4*)(row + k0);
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) dst[i] = (row != nullptr && k0 + i < K) ? row[k0 + i] : (T)0.f;
+    }
+}
+
+// GATE_UP: A rows are gathered token rows, B holds the expert's gate rows and up rows, the epilogue is the activation.
+// else:    A rows are the sorted activation rows, B the expert's down rows, the epilogue weights and scatters.
+template <typename T, int MT, bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_grouped_kernel(
+    const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, const int* __restrict__ sorted_pairs,
+    const int* __restrict__ meta, const float* __restrict__ pair_w, T* __restrict__ y, float* __restrict__ out, int top,
+    int N, int K, float limit, float alpha, int vec_ok) {
+    using M = MoeMma<T>;
+    constexpr int BM = 16 * MT, NB = GATE_UP ? 2 : 1, LD = kMoeBK + M::kPad, KV = kMoeBK / M::kVec;
+    __shared__ __attribute__((aligned(16))) T As[BM * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[NB * kMoeBN * LD];
+    __shared__ int src_row[BM];                    // GATE_UP: token of the row; else the pair of the row; -1 past the tile
+    if ((int)blockIdx.x >= meta[0]) return;
+    const int e = meta[1 + 3 * blockIdx.x], row0 = meta[2 + 3 * blockIdx.x], rows = meta[3 + 3 * blockIdx.x];
+    const int n0 = blockIdx.y * kMoeBN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lq = lane & 15, lg = lane >> 4;
+    for (int i = tid; i < BM; i += 256) {
+        const int pair = i < rows ? sorted_pairs[row0 + i] : -1;
+        src_row[i] = pair < 0 ? -1 : (GATE_UP ? pair / top : pair);
+    }
+    __syncthreads();
+    const T* we = w + (int64_t)e * (NB * (int64_t)N) * K;     // [NB * N, K] of this expert
+    f32x4 acc[NB][MT];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[b][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += kMoeBK) {
+        for (int it = tid; it < BM * KV; it += 256) {
+            const int r = it / KV, kv = (it % KV) * M::kVec;
+            const T* row = nullptr;
+            if (r < rows) row = GATE_UP ? a + (int64_t)src_row[r] * a_stride : a + (int64_t)(row0 + r) * a_stride;
+            moe_stage<T>(As + r * LD + kv, row, k0 + kv, K, vec_ok != 0);
+        }
+        for (int it = tid; it < NB * kMoeBN * KV; it += 256) {
+            const int r = it / KV, kv = (it % KV) * M::kVec;
+            const int n = n0 + (r % kMoeBN);
+            const T* row = n < N ? we + ((int64_t)(r / kMoeBN) * N + n) * K : nullptr;
+            moe_stage<T>(Bs + r * LD + kv, row, k0 + kv, K, vec_ok != 0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < kMoeBK; kk += M::kStep) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const T* brow = Bs + (b * kMoeBN + wave * 16 + lq) * LD + kk;
+#pragma unroll
+                for (int m = 0; m < MT; ++m) acc[b][m] = M::run(As + (m * 16 + lq) * LD + kk, brow, lg, acc[b][m]);
+            }
+        }
+        __syncthreads();
+    }
+    const int n = n0 + wave * 16 + lq;
+    if (n >= N) return;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = m * 16 + 4 * lg + i;
+            if (r >= rows) continue;
+            if constexpr (GATE_UP) {
+                const float g = fminf(acc[0][m][i], limit);
+                const float u = fminf(fmaxf(acc[1][m][i], -limit), limit);
+                y[(int64_t)(row0 + r) * N + n] = (T)(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+            } else {
+                const int pair = src_row[r];
+                out[(int64_t)pair * N + n] = acc[0][m][i] * pair_w[pair];
+            }
+        }
+    }
+}
+
+template <typename T, bool GATE_UP>
+static void launch_grouped(const void* a, int64_t a_stride, const void* w, const int* sorted_pairs, const int* meta,
+                           const float* pair_w, void* y, float* out, int top, int N, int K, float limit, float alpha,
+                           int max_tiles, int tile_rows, hipStream_t s) {
+    const int vec = MoeMma<T>::kVec;
+    const int vec_ok = K % vec == 0 && a_stride % vec == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0;
+    const dim3 grid((unsigned)max_tiles, (unsigned)((N + kMoeBN - 1) / kMoeBN));
+    if (tile_rows == 64)
+        hipLaunchKernelGGL((moe_grouped_kernel<T, 4, GATE_UP>), grid, dim3(256), 0, s, (const T*)a, a_stride, (const T*)w,
+                           sorted_pairs, meta, pair_w, (T*)y, out, top, N, K, limit, alpha, vec_ok);
+    else
+        hipLaunchKernelGGL((moe_grouped_kernel<T, 1, GATE_UP>), grid, dim3(256), 0, s, (const T*)a, a_stride, (const T*)w,
+                           sorted_pairs, meta, pair_w, (T*)y, out, top, N, K, limit, alpha, vec_ok);
+}
+
+}  // namespace nv
+
+extern "C" int nv_moe_route(const float* logits, int32_t* ids, float* weights, int64_t T, int E, int top, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(T >= 0 && E > 0 && top >= 1 && top <= E && top <= kMoeMaxTop, NV_ERR_INVALID_ARG,
+               "nv_moe_route: top=%d must lie in 1 .. min(E=%d, %d)", top, E, kMoeMaxTop);
+    if (T == 0) return NV_OK;
+    NV_REQUIRE(logits && ids && weights, NV_ERR_INVALID_ARG, "nv_moe_route: null pointer");
+    NV_REQUIRE((T + 255) / 256 < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_route: launch too large");
+    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, (hipStream_t)stream, logits, ids,
+                       weights, T, E, top);
+    return check_launch("nv_moe_route");
+}
+
+extern "C" int nv_moe_tile_rows(int64_t pairs, int E) { return pairs >= 32 * (int64_t)E ? 64 : 16; }
+
+extern "C" int64_t nv_moe_max_tiles(int64_t pairs, int E, int tile_rows) {
+    return pairs / tile_rows + std::min<int64_t>(pairs, E);
+}
+
+extern "C" int nv_moe_align(const int32_t* ids, int32_t* sorted_pairs, int32_t* meta, int64_t pairs, int E,
+                            int tile_rows, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(pairs >= 0 && E > 0 && E <= 4096 && (tile_rows == 16 || tile_rows == 64), NV_ERR_INVALID_ARG,
+               "nv_moe_align: bad sizes");
+    NV_REQUIRE(ids && sorted_pairs && meta, NV_ERR_INVALID_ARG, "nv_moe_align: null pointer");
+    NV_REQUIRE(pairs < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_align: too many pairs");
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), sizeof(int) * 2 * (size_t)E, (hipStream_t)stream, ids,
+                       sorted_pairs, meta, pairs, E, tile_rows);
+    return check_launch("nv_moe_align");
+}
+
+extern "C" int nv_moe_gate_up(const void* h, int64_t h_stride, const void* gate_up, const int32_t* sorted_pairs,
+                              const int32_t* meta, void* y, int dtype, int64_t pairs, int E, int top, int width, int ff,
+                              float limit, float alpha, int tile_rows, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(pairs >= 0 && E > 0 && top > 0 && width > 0 && ff > 0 && (tile_rows == 16 || tile_rows == 64),
+               NV_ERR_INVALID_ARG, "nv_moe_gate_up: bad sizes");
+    if (pairs == 0) return NV_OK;
+    NV_REQUIRE(h && gate_up && sorted_pairs && meta && y, NV_ERR_INVALID_ARG, "nv_moe_gate_up: null pointer");
+    NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_moe_gate_up: bad dtype");
+    const int64_t tiles = nv_moe_max_tiles(pairs, E, tile_rows);
+    NV_REQUIRE(tiles < (1LL << 31) && (ff + kMoeBN - 1) / kMoeBN < 65536, NV_ERR_UNSUPPORTED, "nv_moe_gate_up: launch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NV_DTYPE_BF16)
+        launch_grouped<__bf16, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
+                                     alpha, (int)tiles, tile_rows, s);
+    else
+        launch_grouped<float, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
+                                    alpha, (int)tiles, tile_rows, s);
+    return check_launch("nv_moe_gate_up");
+}
+
+extern "C" int nv_moe_down(const void* y, const void* down, const int32_t* sorted_pairs, const int32_t* meta,
+                           const float* pair_weights, float* out, int dtype, int64_t pairs, int E, int width, int ff,
+                           int tile_rows, void* stream) {
+    using namespace nv;
+    NV_REQUIRE(pairs >= 0 && E > 0 && width > 0 && ff > 0 && (tile_rows == 16 || tile_rows == 64), NV_ERR_INVALID_ARG,
+               "nv_moe_down: bad sizes");
+    if (pairs == 0) return NV_OK;
+    NV_REQUIRE(y && down && sorted_pairs && meta && pair_weights && out, NV_ERR_INVALID_ARG, "nv_moe_down: null pointer");
+    NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_moe_down: bad dtype");
+    const int64_t tiles = nv_moe_max_tiles(pairs, E, tile_rows);
+    NV_REQUIRE(tiles < (1LL << 31) && (width + kMoeBN - 1) / kMoeBN < 65536, NV_ERR_UNSUPPORTED, "nv_moe_down: launch too large");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == NV_DTYPE_BF16)
+        launch_grouped<__bf16, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f,
+                                      (int)tiles, tile_rows, s);
+    else
+        launch_grouped<float, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f,
+                                     (int)tiles, tile_rows, s);
+    return check_launch("nv_moe_down");
+}

@@ -563,3 +563,215 @@ def gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a_raw: t
                                  state_slots.data_ptr(), B, H, G, D, Dv, float(eps), dt, _stream(q))
     _lib.check(rc, "nv_gated_delta_rule", dll)
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------
+# fp32 stream with a grouped RMS norm, input convolution, token gate, generalized delta rule, latent attention
+# and routed experts (second library).
+# ---------------------------------------------------------------------------------------------------------
+def stream_boundary(x: torch.Tensor, add: Optional[torch.Tensor] = None, add_parts: Optional[torch.Tensor] = None,
+                    normed: Optional[torch.Tensor] = None, normed_weight: Optional[torch.Tensor] = None,
+                    mult: float = 1.0, norm: Optional[torch.Tensor] = None, groups: int = 1, eps: float = 1e-5,
+                    out_dtype: Optional[torch.dtype] = None, want_f32: bool = False,
+                    copy_dtype: Optional[torch.dtype] = None):
+    """One boundary of an fp32 residual stream, in place on x [T, W]:
+    x += mult * (add + add_parts.sum(1));  x += mult * rmsnorm(normed) * normed_weight  (each part optional).
+    With `norm` (the weight of a grouped RMS norm) returns (h32 or None, h): the norm of x in float32 (if want_f32)
+    and in out_dtype; else with `copy_dtype` returns x in that dtype; else None."""
+    _need(x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(),
+          "the stream must be a contiguous float32 [tokens, width] GPU tensor")
+    rows, cols = x.shape
+    dt_t = out_dtype or copy_dtype or (add.dtype if add is not None else normed.dtype if normed is not None else torch.float32)
+    dt = _lib.DTYPE_BF16 if dt_t == _BF16 else _lib.DTYPE_F32
+    _need(dt_t in (_BF16, torch.float32), "the matmul dtype must be bfloat16 or float32")
+    for t, n in ((add, "add"), (normed, "normed")):
+        if t is not None:
+            _rows2d(t, n)
+            _need(t.shape == x.shape and t.dtype == dt_t and t.is_cuda, f"{n} must match the stream's shape, in the matmul dtype")
+    n_parts = 0
+    if add_parts is not None:
+        _need(add_parts.is_cuda and add_parts.dtype == torch.float32 and add_parts.is_contiguous() and add_parts.dim() == 3
+              and add_parts.shape[0] == rows and add_parts.shape[2] == cols, "add_parts must be contiguous float32 [T, n, W]")
+        n_parts = add_parts.shape[1]
+    if normed is not None:
+        _need(normed_weight is not None and normed_weight.numel() == cols, "normed needs its [width] weight")
+    y32 = y = copy = None
+    if norm is not None:
+        _need(norm.numel() == cols, "norm weight must be [width]")
+        y = torch.empty((rows, cols), dtype=dt_t, device=x.device)
+        if want_f32:
+            y32 = y if dt_t == torch.float32 else torch.empty((rows, cols), dtype=torch.float32, device=x.device)
+    elif copy_dtype is not None:
+        copy = torch.empty((rows, cols), dtype=dt_t, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_stream_boundary(x.data_ptr(), _ptr(add), add.stride(0) if add is not None else 0,
+                                _ptr(add_parts) if n_parts else None, n_parts, _ptr(normed),
+                                normed.stride(0) if normed is not None else 0,
+                                _f32c(normed_weight, "normed_weight") if normed is not None else None, float(mult),
+                                _f32c(norm, "norm") or None, int(groups), float(eps),
+                                _ptr(y32) if (y32 is not None and y32 is not y) else None, _ptr(y), _ptr(copy), dt, rows,
+                                cols, _stream(x))
+    _lib.check(rc, "nv_stream_boundary", dll)
+    if norm is not None:
+        return y32, y
+    return copy
+
+
+def rms_norm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * weight per row (fp32 arithmetic), x [T, C] bfloat16 or float32."""
+    dt = _dt(x, "x")
+    _rows2d(x, "x")
+    _need(weight.numel() == x.shape[1], "weight must be [cols]")
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_rms_norm_rows(x.data_ptr(), x.stride(0), _f32c(weight, "weight"), y.data_ptr(), dt, x.shape[0],
+                              x.shape[1], float(eps), _stream(x))
+    _lib.check(rc, "nv_rms_norm_rows", dll)
+    return y
+
+
+def causal_conv_add(x: torch.Tensor, weight: torch.Tensor, conv_state: torch.Tensor, out_dtype: torch.dtype,
+                    cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, state_slots: torch.Tensor) -> torch.Tensor:
+    """x + causal convolution over time per channel, x [T, C] float32; weight [C, taps] float32; conv_state
+    [num_slots, taps - 1, C] float32 carries each sequence's last inputs and is updated; result in out_dtype."""
+    _need(x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [T, C]")
+    T, Cc = x.shape
+    taps = weight.shape[1]
+    _need(weight.shape[0] == Cc, "weight must be [channels, taps]")
+    _need(conv_state.is_cuda and conv_state.dtype == torch.float32 and conv_state.is_contiguous()
+          and conv_state.shape[1:] == (taps - 1, Cc), "conv_state must be contiguous float32 [slots, taps - 1, C]")
+    for t, n in ((cu_seqlens_q, "cu_seqlens_q"), (cu_seqlens_k, "cu_seqlens_k"), (state_slots, "state_slots")):
+        _i32(t, n)
+    B = state_slots.numel()
+    _need(cu_seqlens_q.numel() == B + 1 and cu_seqlens_k.numel() == B + 1, "one state slot per sequence")
+    y = torch.empty((T, Cc), dtype=out_dtype, device=x.device)
+    dll = _lib.mixers()
+    rc = dll.nv_causal_conv_add(x.data_ptr(), _f32c(weight, "weight"), conv_state.data_ptr() if taps > 1 else None,
+                                y.data_ptr(), _dt(y, "y"), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
+                                state_slots.data_ptr(), B, T, Cc, taps, _stream(x))
+    _lib.check(rc, "nv_causal_conv_add", dll)
+    return y
+
+
+def token_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, offset: int, dim: int) -> torch.Tensor:
+    """gelu_tanh(z) * table[ids, offset : offset + dim]; z [T, dim] and table [V, n] of one dtype."""
+    dt = _dt(z, "z")
+    _rows2d(z, "z")
+    _rows2d(table, "table")
+    _need(table.dtype == z.dtype and table.is_cuda and z.shape[1] == dim and 0 <= offset and offset + dim <= table.shape[1],
+          "table must be of z's dtype and hold the columns offset .. offset + dim")
+    _need(ids.is_cuda and ids.dtype == torch.int64 and ids.is_contiguous() and ids.numel() == z.shape[0],
+          "ids must be a contiguous int64 [tokens] GPU tensor")
+    y = torch.empty((z.shape[0], dim), dtype=z.dtype, device=z.device)
+    dll = _lib.mixers()
+    rc = dll.nv_token_gate(z.data_ptr(), z.stride(0), table.data_ptr(), table.stride(0), ids.data_ptr(), int(offset),
+                           int(dim), y.data_ptr(), dt, z.shape[0], _stream(z))
+    _lib.check(rc, "nv_token_gate", dll)
+    return y
+
+
+def general_delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w_raw: torch.Tensor, a_raw: torch.Tensor,
+                       gate_raw: torch.Tensor, w_bias: torch.Tensor, a_bias: torch.Tensor, norm_weight: torch.Tensor,
+                       state: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
+                       state_slots: torch.Tensor, eps: float, decay_rate: float, key_eps: float) -> torch.Tensor:
+    """Generalized delta rule over a step's rows, state [slots, H, D, D] float32 updated in place; r, k, v: [T, H, D];
+    w_raw, a_raw, gate_raw: [T, H * D]; returns the normalised, gated read-out [T, H * D]."""
+    dt = _dt(r, "r")
+    T, H, D = r.shape
+    for t, n in ((r, "r"), (k, "k"), (v, "v")):
+        _rows_ok(t, n)
+        _need(t.shape == (T, H, D) and t.dtype == r.dtype, "r, k, v must be [T, H, D] of one dtype")
+    for t, n in ((w_raw, "w_raw"), (a_raw, "a_raw"), (gate_raw, "gate_raw")):
+        _rows2d(t, n)
+        _need(t.shape == (T, H * D) and t.dtype == r.dtype, f"{n} must be [T, H * D] of r's dtype")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, D),
+          "state must be contiguous float32 [slots, H, D, D]")
+    _need(w_bias.numel() == H * D and a_bias.numel() == H * D and norm_weight.numel() == H * D, "constant shapes")
+    for t, n in ((cu_seqlens_q, "cu_seqlens_q"), (cu_seqlens_k, "cu_seqlens_k"), (state_slots, "state_slots")):
+        _i32(t, n)
+    B = state_slots.numel()
+    _need(cu_seqlens_q.numel() == B + 1 and cu_seqlens_k.numel() == B + 1, "one state slot per sequence")
+    out = torch.empty((T, H * D), dtype=r.dtype, device=r.device)
+    dll = _lib.mixers()
+    rc = dll.nv_general_delta_rule(r.data_ptr(), k.data_ptr(), v.data_ptr(), r.stride(0), k.stride(0), v.stride(0),
+                                   w_raw.data_ptr(), w_raw.stride(0), a_raw.data_ptr(), a_raw.stride(0),
+                                   gate_raw.data_ptr(), gate_raw.stride(0), _f32c(w_bias, "w_bias"),
+                                   _f32c(a_bias, "a_bias"), _f32c(norm_weight, "norm_weight"), state.data_ptr(),
+                                   out.data_ptr(), out.stride(0), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(),
+                                   state_slots.data_ptr(), B, H, D, float(eps), float(decay_rate), float(key_eps), dt,
+                                   _stream(r))
+    _lib.check(rc, "nv_general_delta_rule", dll)
+    return out
+
+
+def latent_prep_store(q: torch.Tensor, q_lat: torch.Tensor, ckv: torch.Tensor, latent_weight: torch.Tensor,
+                      freq: Optional[torch.Tensor], mag: float, interleaved: bool, positions: torch.Tensor,
+                      slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                      v_cache: Optional[torch.Tensor], rot_dim: int, eps: float) -> torch.Tensor:
+    """Normalises the latent, rotates the shared key part and the queries' rotated part, scatters [c | k_r] and c into
+    the paged caches and returns the latent-space queries [T, H, rank + R].  q: [T, H, Dq] whose last R columns are
+    rotated; q_lat: [T, H, rank] (any token / head strides); ckv: [T, rank + R]."""
+    dt = _dt(q, "q")
+    _rows_ok(q, "q")
+    T, H, Dq = q.shape
+    R, rank = int(rot_dim), q_lat.shape[2]
+    _need(q_lat.shape[:2] == (T, H) and q_lat.stride(2) == 1 and q_lat.dtype == q.dtype and q_lat.is_cuda,
+          "q_lat must be [T, H, rank] of q's dtype with contiguous columns")
+    _rows2d(ckv, "ckv")
+    _need(ckv.shape == (T, rank + R) and ckv.dtype == q.dtype, "ckv must be [T, rank + R] of q's dtype")
+    _need(latent_weight.numel() == rank, "latent weight must be [rank]")
+    _need(positions.is_cuda and positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == T,
+          "positions must be a contiguous int64 [tokens] GPU tensor")
+    if R:
+        _need(freq is not None and freq.numel() == R // 2, "freq must hold R / 2 frequencies")
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "slot_mapping length != number of tokens")
+        _need(k_cache is not None and v_cache is not None and k_cache.is_contiguous() and v_cache.is_contiguous()
+              and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[2:] == (1, rank + R)
+              and v_cache.shape[2:] == (1, rank) and k_cache.shape[:2] == v_cache.shape[:2],
+              "caches must be contiguous [num_blocks, block_size, 1, rank + R] and [.., 1, rank] of q's dtype")
+    q_full = torch.empty((T, H, rank + R), dtype=q.dtype, device=q.device)
+    dll = _lib.mixers()
+    rc = dll.nv_latent_prep_store(q.data_ptr(), q.stride(0), Dq, q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1),
+                                  ckv.data_ptr(), ckv.stride(0), _f32c(latent_weight, "latent_weight"),
+                                  _f32c(freq, "freq") or None, float(mag), int(bool(interleaved)), positions.data_ptr(),
+                                  _ptr(slot_mapping), q_full.data_ptr(), _ptr(k_cache), _ptr(v_cache), dt, T, H, rank, R,
+                                  float(eps), _stream(q))
+    _lib.check(rc, "nv_latent_prep_store", dll)
+    return q_full
+
+
+def moe_experts(h: torch.Tensor, logits: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top: int,
+                limit: float, alpha: float) -> torch.Tensor:
+    """Routed clamped-GLU experts: h [T, W]; logits [T, E] float32; gate_up [E, 2 ff, W]; down [E, W, ff].  Returns the
+    weighted outputs of every token's `top` experts, [T, top, W] float32 (the stream update sums them)."""
+    dt = _dt(h, "h")
+    _rows2d(h, "h")
+    T, W = h.shape
+    E, ff = gate_up.shape[0], gate_up.shape[1] // 2
+    _need(logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and logits.shape == (T, E),
+          "logits must be contiguous float32 [T, E]")
+    _need(gate_up.is_cuda and down.is_cuda and gate_up.is_contiguous() and down.is_contiguous() and gate_up.dtype == h.dtype
+          and down.dtype == h.dtype and gate_up.shape == (E, 2 * ff, W) and down.shape == (E, W, ff),
+          "gate_up must be [E, 2 ff, W] and down [E, W, ff], contiguous, of h's dtype")
+    dll = _lib.mixers()
+    dev, P, s = h.device, T * top, _stream(h)
+    ids = torch.empty((T, top), dtype=torch.int32, device=dev)
+    wgt = torch.empty((T, top), dtype=torch.float32, device=dev)
+    out = torch.empty((T, top, W), dtype=torch.float32, device=dev)
+    if T == 0:
+        return out
+    _lib.check(dll.nv_moe_route(logits.data_ptr(), ids.data_ptr(), wgt.data_ptr(), T, E, int(top), s), "nv_moe_route", dll)
+    rows = dll.nv_moe_tile_rows(P, E)
+    tiles = dll.nv_moe_max_tiles(P, E, rows)
+    sorted_pairs = torch.empty(P, dtype=torch.int32, device=dev)
+    meta = torch.empty(1 + 3 * tiles, dtype=torch.int32, device=dev)
+    _lib.check(dll.nv_moe_align(ids.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), P, E, rows, s), "nv_moe_align", dll)
+    y = torch.empty((P, ff), dtype=h.dtype, device=dev)
+    _lib.check(dll.nv_moe_gate_up(h.data_ptr(), h.stride(0), gate_up.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(),
+                                  y.data_ptr(), dt, P, E, int(top), W, ff, float(limit), float(alpha), rows, s),
+               "nv_moe_gate_up", dll)
+    _lib.check(dll.nv_moe_down(y.data_ptr(), down.data_ptr(), sorted_pairs.data_ptr(), meta.data_ptr(), wgt.data_ptr(),
+                               out.data_ptr(), dt, P, E, W, ff, rows, s), "nv_moe_down", dll)
+    return out
