@@ -138,13 +138,21 @@ def general_delta(h, W, p, m, eps, dtype):
 
 
 # ------------------------------------------------------------------------------------------ feed-forward
-def moe(h, W, p, mlp, dtype):
+def moe(h, W, p, mlp, dtype, margins=None):
     """Router logits in 32-bit; the `top` largest choose the experts, weighted by a softmax over those logits only.
-    Expert: g = min(G h, lim), u = clamp(U h, -lim, lim), down(g * sigmoid(1.702 g) * (u + 1))."""
+    Expert: g = min(G h, lim), u = clamp(U h, -lim, lim), down(g * sigmoid(1.702 g) * (u + 1)).
+    margins: a list that receives, per token, how far the last chosen logit lies above the first one left out, in units
+    of the token's logit spread (infinite when every expert is chosen)."""
     T = h.shape[0]
     top, lim = mlp["router"]["top"], float(mlp["expert"]["limit"])
     z = linear(h.to(dtype).float(), W[p + "router"].float())
     val, idx = z.topk(top, dim=-1)
+    if margins is not None:
+        if top < z.shape[1]:
+            nxt = z.topk(top + 1, dim=-1).values[:, -1]
+            margins.append((val[:, -1] - nxt) / z.std(dim=-1).clamp_min(1e-9))
+        else:
+            margins.append(torch.full((T,), float("inf")))
     wgt = torch.softmax(val, dim=-1)
     out = torch.zeros(T, W[p + "e0.down"].shape[0])
     for t in range(T):
@@ -173,8 +181,9 @@ def layer_runs(cfg):
     return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
 
-def forward(cfg, W, tokens, dtype=torch.float32):
-    """Returns (logits [T, vocab] float32, residual stream after every layer run [runs, T, width])."""
+def forward(cfg, W, tokens, dtype=torch.float32, margins=None):
+    """Returns (logits [T, vocab] float32, residual stream after every layer run [runs, T, width]).
+    margins: a list that receives every run's router margins (see `moe`)."""
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     eps, groups, mult = float(cfg["norm"]["eps"]), int(cfg["norm"]["groups"]), float(cfg["residual_mult"])
     x = W["embed"][tokens].float() * float(cfg["embedding"]["scale"])
@@ -191,7 +200,7 @@ def forward(cfg, W, tokens, dtype=torch.float32):
         else:
             y = latent_attention(hm, W, p + "mix.", L["mixer"], eps, L["type"] == "latent_attention", dtype).float()
         if L.get("mlp") is not None:
-            y = y + moe(h, W, p + "mlp.", L["mlp"], dtype)
+            y = y + moe(h, W, p + "mlp.", L["mlp"], dtype, margins)
         x = x + mult * y
         if cfg.get("token_side"):
             x = x + mult * token_side(x, tokens, W, i, int(cfg["token_side"]["dim"]), eps, dtype)

@@ -72,9 +72,9 @@ def random_checkpoint(cfg: dict, seed: int, rank: int = 4, dtype=torch.bfloat16)
         else:
             R, Dv, qr, kr = m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"]
             t[p + "mix.dq"], t[p + "mix.dq.norm"] = lin(qr, W), rn(qr, std=0.1, mean=1.0)
-            t[p + "mix.uq"] = lin(H * (D + R), qr, 2.0)
+            t[p + "mix.uq"] = lin(H * (D + R), qr)
             t[p + "mix.dkv"], t[p + "mix.dkv.norm"] = lin(kr + R, W, 1.5), rn(kr, std=0.1, mean=1.0)
-            t[p + "mix.uk"], t[p + "mix.uv"] = lin(H * D, kr, 2.0), lin(H * Dv, kr)
+            t[p + "mix.uk"], t[p + "mix.uv"] = lin(H * D, kr), lin(H * Dv, kr)
             t[p + "mix.o"] = lin(W, H * Dv)
         if L["mlp"] is not None:
             E, ff = L["mlp"]["router"]["experts"], L["mlp"]["expert"]["ff"]
@@ -103,3 +103,14 @@ def layer_namespace(device: str):
         return ref_benarax_modules
     from nanovllm_amd.model.benarax import _default_layers
     return _default_layers()
+
+
+def steady_prefix(cfg: dict, tensors: dict, tokens, least=0.05) -> int:
+    """Number of leading positions before the first close call of a router (the last chosen expert leads the next one
+    by less than `least` of the logits' spread): up to there a bfloat16 run differs from float32 by rounding alone."""
+    margins = []
+    ref_benarax.forward(cfg, tensors, tokens, torch.float32, margins)
+    if not margins:
+        return len(tokens)
+    close = torch.stack(margins).min(0).values < least
+    return int(close.nonzero()[0]) if close.any() else len(tokens)

@@ -10,7 +10,7 @@ import pytest
 import torch
 from safetensors.torch import save_file
 
-from benarax_util import config, delta_layer, latent_layer, moe, oracle_logits, random_checkpoint, rel_err
+from benarax_util import config, delta_layer, latent_layer, moe, oracle_logits, random_checkpoint, rel_err, steady_prefix
 from conftest import ROOT
 from nanovllm_amd.engine.llm_engine import LLMEngine
 from nanovllm_amd.model import registry
@@ -75,15 +75,20 @@ def test_trace_run_replays_steps_and_writes_logits(tmp_path, dtype):
     assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
     V = CFG["vocab"]
     la, lb = oracle_logits(CFG, ck, a), oracle_logits(CFG, ck, b)
-    want = {0: [la[0], la[16]], 1: [lb[5]], 2: [lb[6], la[19 + 20], la[19]], 3: [lb[6]]}
-    bound = 5e-5 if dtype == "float32" else 3 * max(rel_err(oracle_logits(CFG, ck, a, torch.bfloat16), la),
-                                                    rel_err(oracle_logits(CFG, ck, b, torch.bfloat16), lb))
+    want = {0: [("a", 0), ("a", 16)], 1: [("b", 5)], 2: [("b", 6), ("a", 19 + 20), ("a", 19)], 3: [("b", 6)]}
+    ref = {"a": la, "b": lb}
+    # bfloat16: rounding-sized bound, on positions before a router's first close call (see steady_prefix)
+    steady = {"a": len(a), "b": len(b)} if dtype == "float32" else {"a": steady_prefix(CFG, ck, a), "b": steady_prefix(CFG, ck, b)}
+    bound = 5e-5 if dtype == "float32" else 3 * max(rel_err(oracle_logits(CFG, ck, a, torch.bfloat16)[:max(steady["a"], 1)], la[:max(steady["a"], 1)]),
+                                                    rel_err(oracle_logits(CFG, ck, b, torch.bfloat16)[:max(steady["b"], 1)], lb[:max(steady["b"], 1)]))
     for n, rows in want.items():
         got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{n}.f32"), dtype="<f4").reshape(-1, V).copy())
         assert got.shape[0] == len(rows)
         scale = la.pow(2).mean().sqrt()
-        for g, w in zip(got, rows):
-            d = g - w
+        for g, (i, at) in zip(got, rows):
+            if at >= steady[i]:
+                continue
+            d = g - ref[i][at]
             assert ((d - d.mean()).pow(2).mean().sqrt() / scale).item() < bound, (n, dtype)
 
 
