@@ -65,6 +65,9 @@ def parse():
     ap.add_argument("--buvalix", action="store_true",
                     help="instead of the default workload: the Buvalix kernels and model beside the Qwen3 path at "
                          "equal sizes (one GPU, random weights), one JSON line")
+    ap.add_argument("--benarax", action="store_true",
+                    help="instead of the default workload: the Benarax kernels and model beside Buvalix at equal sizes "
+                         "(one GPU, random weights), one JSON line")
     return ap.parse_args()
 
 
@@ -790,6 +793,12 @@ def main():
             raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
         from tools.buvalix_bench import run as buvalix_run
         print(json.dumps(buvalix_run("cuda:0")))
+        return
+    if args.benarax:
+        if not torch.cuda.is_available():
+            raise SystemExit("bench.py needs a GPU (the hot path has no CPU implementation)")
+        from tools.benarax_bench import run as benarax_run
+        print(json.dumps(benarax_run("cuda:0")))
         return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -62,7 +62,7 @@ NV_API int nv_qk_prep_store(const void* q, const void* k, const void* v, void* q
  * k_cache: [num_blocks, block_size, G, D], v_cache: [num_blocks, block_size, G, Dv]; query i of sequence b sits at
  * position len_k(b) - len_q(b) + i.  Dv <= 256.
  * max_seqlen_q / max_seqlen_k: the most rows / keys any sequence has in this step (0 = unknown).  Three kernels
- * share the work: sequences with several rows run on a bf16 MFMA tile kernel (head sizes in multiples of 16) sized from
+ * share the work: sequences with several rows run on a bf16 MFMA tile kernel (head sizes: multiples of 16 up to 128, of 32 up to 320 / 256) sized from
  * max_seqlen_q; sequences with one row on a decode kernel that reads K/V once per group of query heads and cuts long
  * contexts into key slices (planned from max_seqlen_k, joined through `workspace`); whatever shape neither takes
  * runs one row per wave.  single_rows = 0 promises that no sequence has exactly one row; max_seqlen_q = 1 that all do.

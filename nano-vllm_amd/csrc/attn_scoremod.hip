@@ -230,7 +230,9 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
     // its key's K row and V row.  One block-table lookup per thread and tile, every load of a tile issued before
     // anything waits on one, and the next tile's loads are in flight while this tile is computed.
     const int my_key = tid & (kTileK - 1), my_quarter = tid >> 6;
-    constexpr int KP = DS / 2, VP = DVS / 2;                    // 16-byte pieces per thread of a K row / a V row
+    // 16-byte pieces per thread of a K row / a V row (a row has 2 DS / 2 DVS pieces; with an odd count the last round
+    // is taken by the first two quarters only)
+    constexpr int KP = (2 * DS + 3) / 4, VP = (2 * DVS + 3) / 4;
     uint4 kreg[KP], vreg[VP];
     auto fetch = [&](int base) {
         const int j = base + my_key;
@@ -239,16 +241,19 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
         if (in) row = ((int64_t)table[j / block_size] * block_size + (j % block_size)) * G + g;
 #pragma unroll
         for (int i = 0; i < KP; ++i)
-            kreg[i] = in ? *(const uint4*)(k_cache + row * D + 8 * (my_quarter + 4 * i)) : make_uint4(0, 0, 0, 0);
+            kreg[i] = (in && my_quarter + 4 * i < 2 * DS) ? *(const uint4*)(k_cache + row * D + 8 * (my_quarter + 4 * i))
+                                                         : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < VP; ++i)
-            vreg[i] = in ? *(const uint4*)(v_cache + row * Dv + 8 * (my_quarter + 4 * i)) : make_uint4(0, 0, 0, 0);
+            vreg[i] = (in && my_quarter + 4 * i < 2 * DVS) ? *(const uint4*)(v_cache + row * Dv + 8 * (my_quarter + 4 * i))
+                                                          : make_uint4(0, 0, 0, 0);
     };
     fetch(0);
     for (int base = 0; base <= last_pos; base += kTileK) {
         __syncthreads();                                      // the previous tile has been consumed
 #pragma unroll
         for (int i = 0; i < KP; ++i) {                        // rows are 8-byte aligned: two 8-byte stores
+            if (my_quarter + 4 * i >= 2 * DS) continue;
             uint2* dst = (uint2*)(ldsK + my_key * k_ld + 8 * (my_quarter + 4 * i));
             dst[0] = make_uint2(kreg[i].x, kreg[i].y);
             dst[1] = make_uint2(kreg[i].z, kreg[i].w);
@@ -258,6 +263,7 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
             // V goes in transposed; consecutive lanes hold consecutive keys, so each of the eight 2-byte stores of a
             // wave lands in consecutive LDS words
             const int ch = my_quarter + 4 * i;
+            if (ch >= 2 * DVS) continue;
             const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -632,6 +638,54 @@ extern "C" int64_t nv_attn_scoremod_workspace_bytes(int num_seqs, int64_t T, int
     return nv::decode_plan(num_seqs, T, H, G, Dv, max_seqlen_k).ws_bytes;
 }
 
+namespace nv {
+// Head sizes the tile kernel is built for: every multiple of 16 up to 128, every multiple of 32 up to 320.
+static bool tile_built(int n) { return n >= 32 && n % 16 == 0 && (n <= 128 || n % 32 == 0); }
+struct TileArgs {
+    const __bf16 *q, *k_cache, *v_cache;
+    __bf16* out;
+    const int *cu_q, *cu_k, *block_tables;
+    int max_blocks, tiles, H, G, D, Dv, block_size;
+    float scale, softcap;
+    const float *sink, *dist_bias;
+    int n_dist;
+    int64_t q_stride, out_stride;
+};
+template <int DS, int DVS>
+static bool launch_tile_one(dim3 grid, size_t lds, hipStream_t s, const TileArgs& a) {
+    if (lds > 64 * 1024) {      // more than the default limit of dynamic LDS: raise this instantiation's once
+        static bool raised = false;
+        if (!raised) {
+            if (hipFuncSetAttribute((const void*)attn_scoremod_tile_kernel<DS, DVS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    80 * 1024) != hipSuccess)
+                return false;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL((attn_scoremod_tile_kernel<DS, DVS>), grid, dim3(kTileThreads), lds, s, a.q, a.k_cache, a.v_cache, a.out,
+                       a.cu_q, a.cu_k, a.block_tables, a.max_blocks, a.tiles, a.H, a.G, a.D, a.Dv, a.block_size, a.scale,
+                       a.softcap, a.sink, a.dist_bias, a.n_dist, a.q_stride, a.out_stride);
+    return true;
+}
+template <int DS>
+static bool launch_tile_dv(int dvs, dim3 grid, size_t lds, hipStream_t s, const TileArgs& a) {
+    switch (dvs) {
+#define NV_DV(N) case N: return launch_tile_one<DS, N>(grid, lds, s, a);
+        NV_DV(2) NV_DV(3) NV_DV(4) NV_DV(5) NV_DV(6) NV_DV(7) NV_DV(8) NV_DV(10) NV_DV(12) NV_DV(14) NV_DV(16)
+#undef NV_DV
+    }
+    return false;
+}
+static bool launch_tile(int ds, int dvs, dim3 grid, size_t lds, hipStream_t s, const TileArgs& a) {
+    switch (ds) {
+#define NV_D(N) case N: return launch_tile_dv<N>(dvs, grid, lds, s, a);
+        NV_D(2) NV_D(3) NV_D(4) NV_D(5) NV_D(6) NV_D(7) NV_D(8) NV_D(10) NV_D(12) NV_D(14) NV_D(16) NV_D(18) NV_D(20)
+#undef NV_D
+    }
+    return false;
+}
+}  // namespace nv
+
 extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const void* v_cache, void* out,
                                       const int* cu_seqlens_q, const int* cu_seqlens_k, const int* block_tables,
                                       int num_seqs, int max_blocks_per_seq, int64_t T, int H, int G, int D, int Dv,
@@ -656,10 +710,11 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     hipStream_t s = (hipStream_t)stream;
     const bool bf = dtype == NV_DTYPE_BF16;
     const bool several = max_seqlen_q != 1, singles = single_rows != 0;      // what the step may hold
-    // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes 32, 64, 96 or 128, aligned rows), else the row-per-wave kernel.
+    // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes in built multiples of
+    // 16, aligned rows), else the row-per-wave kernel.
     const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 4) + (size_t)Dv * (kTileK + 4));
-    const auto tile_size = [](int n) { return n == 32 || n == 64 || n == 96 || n == 128; };      // built tile shapes
-    const bool tile_ok = bf && max_seqlen_q > 1 && tile_size(D) && tile_size(Dv) && tile_lds <= 64 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
+    const bool tile_ok = bf && max_seqlen_q > 1 && tile_built(D) && tile_built(Dv) && D <= 320 && Dv <= 256 &&
+                         tile_lds <= 80 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
                          ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
     // Sequences with one row: the decode kernel (key slices, the query heads of a group together) when rows can be
     // read in 16-byte pieces, else the row-per-wave kernel.
@@ -676,18 +731,11 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
         const int tiles = (max_seqlen_q + kTileQ - 1) / kTileQ;
         NV_REQUIRE((int64_t)num_seqs * tiles < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_attn_scoremod_paged: launch too large");
         const dim3 tgrid((unsigned)(num_seqs * tiles), (unsigned)H);
-#define NV_TILE_ARGS                                                                                                  \
-    (const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q, cu_seqlens_k,      \
-        block_tables, max_blocks_per_seq, tiles, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,  \
-        q_stride, out_stride
-#define NV_TILE_CASE(A, B)                                                                                          \
-    if (D == 16 * A && Dv == 16 * B)                                                                                \
-        hipLaunchKernelGGL((attn_scoremod_tile_kernel<A, B>), tgrid, dim3(kTileThreads), tile_lds, s, NV_TILE_ARGS);
-#define NV_TILE_ROW(A) NV_TILE_CASE(A, 2) NV_TILE_CASE(A, 4) NV_TILE_CASE(A, 6) NV_TILE_CASE(A, 8)
-        NV_TILE_ROW(2) NV_TILE_ROW(4) NV_TILE_ROW(6) NV_TILE_ROW(8)
-#undef NV_TILE_ROW
-#undef NV_TILE_CASE
-#undef NV_TILE_ARGS
+        const TileArgs ta{(const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q,
+                          cu_seqlens_k, block_tables, max_blocks_per_seq, tiles, H, G, D, Dv, block_size, scale, softcap,
+                          sink, dist_bias, n_dist, q_stride, out_stride};
+        NV_REQUIRE(launch_tile(D / 16, Dv / 16, tgrid, tile_lds, s, ta), NV_ERR_LAUNCH,
+                   "nv_attn_scoremod_paged: no tile kernel for D=%d, Dv=%d", D, Dv);
         const int rc = check_launch("nv_attn_scoremod_paged (tile kernel)");
         if (rc != NV_OK) return rc;
     }

@@ -11,8 +11,8 @@
 //                       the `top` rows of a token in a fixed order (no atomics, bitwise reproducible).
 //
 // Both products are one grouped matrix product on the matrix cores: a workgroup of four waves takes one row tile
-// (16 or 64 rows of ONE expert) and 64 output columns, stages 32-deep slices of the rows and of the expert's weight
-// rows through LDS and issues v_mfma_f32_16x16x16_bf16 (bfloat16) or v_mfma_f32_16x16x4_f32 (true fp32) on them; a
+// (16 or 64 rows of ONE expert) and 64 output columns, stages 64-deep (fp32: 32-deep) slices of the rows and of the
+// expert's weight rows through LDS, the next slices already on their way into registers, and issues v_mfma_f32_16x16x16_bf16 (bfloat16) or v_mfma_f32_16x16x4_f32 (true fp32) on them; a
 // wave owns 16 columns and all row sub-tiles, so every weight element is read from LDS once per 16 rows.  Weights are
 // [E, rows_out, rows_in] with the contraction index contiguous, as stored.  The launch is sized for the most tiles any
 // routing can produce; workgroups beyond the table's count return at once.
@@ -24,7 +24,7 @@
 namespace nv {
 
 constexpr int kMoeMaxTop = 16;
-constexpr int kMoeBN = 64, kMoeBK = 32;
+constexpr int kMoeBN = 64;
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int* __restrict__ ids,
                                                         float* __restrict__ wgt, int64_t T, int E, int top) {
@@ -89,39 +89,41 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
 
 template <typename T> struct MoeMma;
 template <> struct MoeMma<__bf16> {
-    static constexpr int kVec = 8, kPad = 8, kStep = 16;
+    static constexpr int kVec = 8, kPad = 8, kStep = 16, kBK = 64;
     static __device__ __forceinline__ f32x4 run(const __bf16* a, const __bf16* b, int lg, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*(const s16x4*)(a + 4 * lg), *(const s16x4*)(b + 4 * lg), c, 0, 0, 0);
     }
 };
 template <> struct MoeMma<float> {
-    static constexpr int kVec = 4, kPad = 4, kStep = 4;
+    static constexpr int kVec = 4, kPad = 4, kStep = 4, kBK = 32;
     static __device__ __forceinline__ f32x4 run(const float* a, const float* b, int lg, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x4f32(a[lg], b[lg], c, 0, 0, 0);
     }
 };
 
-// kVec elements of a row starting at k0 into LDS, zeros past K (or for a missing row)
+// 16 bytes (kVec elements) of a row starting at k0, zeros past K or for a missing row
 template <typename T>
-__device__ __forceinline__ void moe_stage(T* dst, const T* row, int k0, int K, bool vec_ok) {
+__device__ __forceinline__ uint4 moe_fetch(const T* row, int k0, int K, bool vec_ok) {
     constexpr int V = MoeMma<T>::kVec;
-    if (row != nullptr && vec_ok && k0 + V <= K) {
-        *(uint4*)dst = *(const uint4*)(row + k0);
-    } else {
+    if (row == nullptr || k0 >= K) return make_uint4(0, 0, 0, 0);
+    if (vec_ok && k0 + V <= K) return *(const uint4*)(row + k0);
+    __attribute__((aligned(16))) T tmp[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) dst[i] = (row != nullptr && k0 + i < K) ? row[k0 + i] : (T)0.f;
-    }
+    for (int i = 0; i < V; ++i) tmp[i] = k0 + i < K ? row[k0 + i] : (T)0.f;
+    return *(const uint4*)tmp;
 }
 
 // GATE_UP: A rows are gathered token rows, B holds the expert's gate rows and up rows, the epilogue is the activation.
 // else:    A rows are the sorted activation rows, B the expert's down rows, the epilogue weights and scatters.
+// The slices of the next step are fetched into registers while the current ones are multiplied out of LDS.
 template <typename T, int MT, bool GATE_UP>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, const int* __restrict__ sorted_pairs,
     const int* __restrict__ meta, const float* __restrict__ pair_w, T* __restrict__ y, float* __restrict__ out, int top,
     int N, int K, float limit, float alpha, int vec_ok) {
     using M = MoeMma<T>;
-    constexpr int BM = 16 * MT, NB = GATE_UP ? 2 : 1, LD = kMoeBK + M::kPad, KV = kMoeBK / M::kVec;
+    constexpr int BK = M::kBK, BM = 16 * MT, NB = GATE_UP ? 2 : 1, LD = BK + M::kPad, KV = BK / M::kVec;
+    constexpr int A_IT = (BM * KV + 255) / 256, B_IT = (NB * kMoeBN * KV + 255) / 256;
     __shared__ __attribute__((aligned(16))) T As[BM * LD];
     __shared__ __attribute__((aligned(16))) T Bs[NB * kMoeBN * LD];
     __shared__ int src_row[BM];                    // GATE_UP: token of the row; else the pair of the row; -1 past the tile
@@ -135,27 +137,49 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     }
     __syncthreads();
     const T* we = w + (int64_t)e * (NB * (int64_t)N) * K;     // [NB * N, K] of this expert
+    // what this thread stages: row pointers are fixed over the K loop
+    const T* a_row[A_IT];
+    const T* b_row[B_IT];
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+        const int it = tid + 256 * i, r = it / KV;
+        a_row[i] = nullptr;
+        if (it < BM * KV && r < rows) a_row[i] = GATE_UP ? a + (int64_t)src_row[r] * a_stride : a + (int64_t)(row0 + r) * a_stride;
+    }
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+        const int it = tid + 256 * i, r = it / KV, n = n0 + (r % kMoeBN);
+        b_row[i] = (it < NB * kMoeBN * KV && n < N) ? we + ((int64_t)(r / kMoeBN) * N + n) * K : nullptr;
+    }
+    uint4 a_reg[A_IT], b_reg[B_IT];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) a_reg[i] = moe_fetch<T>(a_row[i], k0 + ((tid + 256 * i) % KV) * M::kVec, K, vec_ok != 0);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) b_reg[i] = moe_fetch<T>(b_row[i], k0 + ((tid + 256 * i) % KV) * M::kVec, K, vec_ok != 0);
+    };
     f32x4 acc[NB][MT];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[b][m] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += kMoeBK) {
-        for (int it = tid; it < BM * KV; it += 256) {
-            const int r = it / KV, kv = (it % KV) * M::kVec;
-            const T* row = nullptr;
-            if (r < rows) row = GATE_UP ? a + (int64_t)src_row[r] * a_stride : a + (int64_t)(row0 + r) * a_stride;
-            moe_stage<T>(As + r * LD + kv, row, k0 + kv, K, vec_ok != 0);
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        __syncthreads();                               // the previous slices have been consumed
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) {
+            const int it = tid + 256 * i;
+            if (it < BM * KV) *(uint4*)(As + (it / KV) * LD + (it % KV) * M::kVec) = a_reg[i];
         }
-        for (int it = tid; it < NB * kMoeBN * KV; it += 256) {
-            const int r = it / KV, kv = (it % KV) * M::kVec;
-            const int n = n0 + (r % kMoeBN);
-            const T* row = n < N ? we + ((int64_t)(r / kMoeBN) * N + n) * K : nullptr;
-            moe_stage<T>(Bs + r * LD + kv, row, k0 + kv, K, vec_ok != 0);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) {
+            const int it = tid + 256 * i;
+            if (it < NB * kMoeBN * KV) *(uint4*)(Bs + (it / KV) * LD + (it % KV) * M::kVec) = b_reg[i];
         }
         __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);
 #pragma unroll
-        for (int kk = 0; kk < kMoeBK; kk += M::kStep) {
+        for (int kk = 0; kk < BK; kk += M::kStep) {
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const T* brow = Bs + (b * kMoeBN + wave * 16 + lq) * LD + kk;
@@ -163,7 +187,6 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
                 for (int m = 0; m < MT; ++m) acc[b][m] = M::run(As + (m * 16 + lq) * LD + kk, brow, lg, acc[b][m]);
             }
         }
-        __syncthreads();
     }
     const int n = n0 + wave * 16 + lq;
     if (n >= N) return;
