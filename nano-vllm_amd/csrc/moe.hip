@@ -11,9 +11,9 @@
 //                       the `top` rows of a token in a fixed order (no atomics, bitwise reproducible).
 //
 // Both products are one grouped matrix product on the matrix cores: a workgroup of four waves takes one row tile
-// (16 or 64 rows of ONE expert) and 64 output columns, stages 64-deep (fp32: 32-deep) slices of the rows and of the
-// expert's weight rows through LDS, the next slices already on their way into registers, and issues v_mfma_f32_16x16x16_bf16 (bfloat16) or v_mfma_f32_16x16x4_f32 (true fp32) on them; a
-// wave owns 16 columns and all row sub-tiles, so every weight element is read from LDS once per 16 rows.  Weights are
+// (16 or 64 rows of ONE expert) and 64 or 128 output columns, stages 64-deep (fp32: 32-deep) slices of the rows and of the
+// expert's weight rows through LDS, the next slices already on their way into registers, and issues v_mfma_f32_16x16x32_bf16 (bfloat16) or v_mfma_f32_16x16x4_f32 (true fp32) on them; a
+// wave owns 16 or 32 columns and all row sub-tiles.  Weights are
 // [E, rows_out, rows_in] with the contraction index contiguous, as stored.  The launch is sized for the most tiles any
 // routing can produce; workgroups beyond the table's count return at once.
 #include <algorithm>
@@ -89,9 +89,10 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
 
 template <typename T> struct MoeMma;
 template <> struct MoeMma<__bf16> {
-    static constexpr int kVec = 8, kPad = 8, kStep = 16, kBK = 64;
+    static constexpr int kVec = 8, kPad = 8, kStep = 32, kBK = 64;
+    // the 32-deep product of gfx950: a lane holds 8 consecutive k of its row (16-byte LDS reads)
     static __device__ __forceinline__ f32x4 run(const __bf16* a, const __bf16* b, int lg, f32x4 c) {
-        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*(const s16x4*)(a + 4 * lg), *(const s16x4*)(b + 4 * lg), c, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8*)(a + 8 * lg), *(const bf16x8*)(b + 8 * lg), c, 0, 0, 0);
     }
 };
 template <> struct MoeMma<float> {
@@ -116,20 +117,26 @@ __device__ __forceinline__ uint4 moe_fetch(const T* row, int k0, int K, bool vec
 // GATE_UP: A rows are gathered token rows, B holds the expert's gate rows and up rows, the epilogue is the activation.
 // else:    A rows are the sorted activation rows, B the expert's down rows, the epilogue weights and scatters.
 // The slices of the next step are fetched into registers while the current ones are multiplied out of LDS.
-template <typename T, int MT, bool GATE_UP>
+template <typename T, int MT, int NT, bool GATE_UP>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(
     const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, const int* __restrict__ sorted_pairs,
     const int* __restrict__ meta, const float* __restrict__ pair_w, T* __restrict__ y, float* __restrict__ out, int top,
-    int N, int K, float limit, float alpha, int vec_ok) {
+    int N, int K, float limit, float alpha, int vec_ok, int max_tiles) {
     using M = MoeMma<T>;
-    constexpr int BK = M::kBK, BM = 16 * MT, NB = GATE_UP ? 2 : 1, LD = BK + M::kPad, KV = BK / M::kVec;
-    constexpr int A_IT = (BM * KV + 255) / 256, B_IT = (NB * kMoeBN * KV + 255) / 256;
+    constexpr int BK = M::kBK, BM = 16 * MT, BN = 64 * NT, NB = GATE_UP ? 2 : 1, LD = BK + M::kPad, KV = BK / M::kVec;
+    constexpr int A_IT = (BM * KV + 255) / 256, B_IT = (NB * BN * KV + 255) / 256;
     __shared__ __attribute__((aligned(16))) T As[BM * LD];
-    __shared__ __attribute__((aligned(16))) T Bs[NB * kMoeBN * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[NB * BN * LD];
     __shared__ int src_row[BM];                    // GATE_UP: token of the row; else the pair of the row; -1 past the tile
-    if ((int)blockIdx.x >= meta[0]) return;
-    const int e = meta[1 + 3 * blockIdx.x], row0 = meta[2 + 3 * blockIdx.x], rows = meta[3 + 3 * blockIdx.x];
-    const int n0 = blockIdx.y * kMoeBN;
+    // Workgroups go to the chip's 8 XCDs (each with its own L2) round robin by their index: index i runs item
+    // (i % 8) * (items / 8) + i / 8, so one XCD works through neighbouring row tiles -- the tiles of one expert, which
+    // share their weight slices in that L2.  Items: row tile fastest, then the column block.
+    const int items = gridDim.x, per_xcd = items / 8;
+    int item = blockIdx.x;
+    if (item < per_xcd * 8) item = (item % 8) * per_xcd + item / 8;
+    const int tile = item % max_tiles, n0 = (item / max_tiles) * BN;
+    if (tile >= meta[0]) return;
+    const int e = meta[1 + 3 * tile], row0 = meta[2 + 3 * tile], rows = meta[3 + 3 * tile];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lq = lane & 15, lg = lane >> 4;
     for (int i = tid; i < BM; i += 256) {
         const int pair = i < rows ? sorted_pairs[row0 + i] : -1;
@@ -148,8 +155,8 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
     }
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
-        const int it = tid + 256 * i, r = it / KV, n = n0 + (r % kMoeBN);
-        b_row[i] = (it < NB * kMoeBN * KV && n < N) ? we + ((int64_t)(r / kMoeBN) * N + n) * K : nullptr;
+        const int it = tid + 256 * i, r = it / KV, n = n0 + (r % BN);
+        b_row[i] = (it < NB * BN * KV && n < N) ? we + ((int64_t)(r / BN) * N + n) * K : nullptr;
     }
     uint4 a_reg[A_IT], b_reg[B_IT];
     auto fetch = [&](int k0) {
@@ -158,9 +165,9 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) b_reg[i] = moe_fetch<T>(b_row[i], k0 + ((tid + 256 * i) % KV) * M::kVec, K, vec_ok != 0);
     };
-    f32x4 acc[NB][MT];
+    f32x4 acc[NB * NT][MT];
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+    for (int b = 0; b < NB * NT; ++b)
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[b][m] = f32x4{0.f, 0.f, 0.f, 0.f};
     fetch(0);
@@ -174,35 +181,38 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) {
             const int it = tid + 256 * i;
-            if (it < NB * kMoeBN * KV) *(uint4*)(Bs + (it / KV) * LD + (it % KV) * M::kVec) = b_reg[i];
+            if (it < NB * BN * KV) *(uint4*)(Bs + (it / KV) * LD + (it % KV) * M::kVec) = b_reg[i];
         }
         __syncthreads();
         if (k0 + BK < K) fetch(k0 + BK);
 #pragma unroll
         for (int kk = 0; kk < BK; kk += M::kStep) {
 #pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                const T* brow = Bs + (b * kMoeBN + wave * 16 + lq) * LD + kk;
+            for (int b = 0; b < NB * NT; ++b) {      // b = (gate | up) * NT + column sub-tile of this wave
+                const T* brow = Bs + ((b / NT) * BN + (wave * NT + b % NT) * 16 + lq) * LD + kk;
 #pragma unroll
                 for (int m = 0; m < MT; ++m) acc[b][m] = M::run(As + (m * 16 + lq) * LD + kk, brow, lg, acc[b][m]);
             }
         }
     }
-    const int n = n0 + wave * 16 + lq;
-    if (n >= N) return;
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n = n0 + (wave * NT + nt) * 16 + lq;
+        if (n >= N) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = m * 16 + 4 * lg + i;
-            if (r >= rows) continue;
-            if constexpr (GATE_UP) {
-                const float g = fminf(acc[0][m][i], limit);
-                const float u = fminf(fmaxf(acc[1][m][i], -limit), limit);
-                y[(int64_t)(row0 + r) * N + n] = (T)(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
-            } else {
-                const int pair = src_row[r];
-                out[(int64_t)pair * N + n] = acc[0][m][i] * pair_w[pair];
+        for (int m = 0; m < MT; ++m) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = m * 16 + 4 * lg + i;
+                if (r >= rows) continue;
+                if constexpr (GATE_UP) {
+                    const float g = fminf(acc[nt][m][i], limit);
+                    const float u = fminf(fmaxf(acc[NT + nt][m][i], -limit), limit);
+                    y[(int64_t)(row0 + r) * N + n] = (T)(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+                } else {
+                    const int pair = src_row[r];
+                    out[(int64_t)pair * N + n] = acc[nt][m][i] * pair_w[pair];
+                }
             }
         }
     }
@@ -214,13 +224,16 @@ static void launch_grouped(const void* a, int64_t a_stride, const void* w, const
                            int max_tiles, int tile_rows, hipStream_t s) {
     const int vec = MoeMma<T>::kVec;
     const int vec_ok = K % vec == 0 && a_stride % vec == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0;
-    const dim3 grid((unsigned)max_tiles, (unsigned)((N + kMoeBN - 1) / kMoeBN));
-    if (tile_rows == 64)
-        hipLaunchKernelGGL((moe_grouped_kernel<T, 4, GATE_UP>), grid, dim3(256), 0, s, (const T*)a, a_stride, (const T*)w,
-                           sorted_pairs, meta, pair_w, (T*)y, out, top, N, K, limit, alpha, vec_ok);
-    else
-        hipLaunchKernelGGL((moe_grouped_kernel<T, 1, GATE_UP>), grid, dim3(256), 0, s, (const T*)a, a_stride, (const T*)w,
-                           sorted_pairs, meta, pair_w, (T*)y, out, top, N, K, limit, alpha, vec_ok);
+    // many rows per expert: 64 x 128 tiles (a wave owns 32 columns; 128-row tiles measured slower: one workgroup per CU);
+    // few: 16 x 64 tiles, more workgroups per weight byte
+#define NV_MOE_LAUNCH(MT, NT)                                                                                          \
+    hipLaunchKernelGGL((moe_grouped_kernel<T, MT, NT, GATE_UP>), dim3((unsigned)(max_tiles * ((N + 64 * NT - 1) / (64 * NT)))), \
+                       dim3(256), 0, s, (const T*)a, a_stride, (const T*)w, sorted_pairs, meta, pair_w, (T*)y, out, top, N, K,  \
+                       limit, alpha, vec_ok, max_tiles)
+    if (tile_rows == 64 && sizeof(T) == 2) NV_MOE_LAUNCH(4, 2);
+    else if (tile_rows == 64) NV_MOE_LAUNCH(4, 1);
+    else NV_MOE_LAUNCH(1, 1);
+#undef NV_MOE_LAUNCH
 }
 
 }  // namespace nv
@@ -265,7 +278,7 @@ extern "C" int nv_moe_gate_up(const void* h, int64_t h_stride, const void* gate_
     NV_REQUIRE(h && gate_up && sorted_pairs && meta && y, NV_ERR_INVALID_ARG, "nv_moe_gate_up: null pointer");
     NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_moe_gate_up: bad dtype");
     const int64_t tiles = nv_moe_max_tiles(pairs, E, tile_rows);
-    NV_REQUIRE(tiles < (1LL << 31) && (ff + kMoeBN - 1) / kMoeBN < 65536, NV_ERR_UNSUPPORTED, "nv_moe_gate_up: launch too large");
+    NV_REQUIRE(tiles * ((ff + kMoeBN - 1) / kMoeBN) < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_gate_up: launch too large");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == NV_DTYPE_BF16)
         launch_grouped<__bf16, true>(h, h_stride, gate_up, sorted_pairs, meta, nullptr, y, nullptr, top, ff, width, limit,
@@ -286,7 +299,7 @@ extern "C" int nv_moe_down(const void* y, const void* down, const int32_t* sorte
     NV_REQUIRE(y && down && sorted_pairs && meta && pair_weights && out, NV_ERR_INVALID_ARG, "nv_moe_down: null pointer");
     NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_moe_down: bad dtype");
     const int64_t tiles = nv_moe_max_tiles(pairs, E, tile_rows);
-    NV_REQUIRE(tiles < (1LL << 31) && (width + kMoeBN - 1) / kMoeBN < 65536, NV_ERR_UNSUPPORTED, "nv_moe_down: launch too large");
+    NV_REQUIRE(tiles * ((width + kMoeBN - 1) / kMoeBN) < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_down: launch too large");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == NV_DTYPE_BF16)
         launch_grouped<__bf16, false>(y, ff, down, sorted_pairs, meta, pair_weights, nullptr, out, 1, width, ff, 0.f, 0.f,
