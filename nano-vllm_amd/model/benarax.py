@@ -228,9 +228,10 @@ class BenaraxMoE(nn.Module):
         self.down = nn.Parameter(torch.zeros(c.experts, width, c.ff, dtype=dtype, device=device))
         self.experts = L.MoEExperts(c.top, c.limit)
 
-    def forward(self, h):
-        """Returns the weighted expert outputs [T, top, width] float32; the stream update sums them."""
-        logits = F.linear(h.float(), self.router)
+    def forward(self, h, h32=None):
+        """Returns the weighted expert outputs [T, top, width] float32; the stream update sums them.  The router reads
+        the norm's float32 output where the step has it (h32), else h widened."""
+        logits = F.linear(h32 if h32 is not None else h.float(), self.router)
         return self.experts(h, logits, self.gate_up, self.down)
 
 
@@ -386,7 +387,7 @@ class BenaraxForCausalLM(nn.Module):
             conv_state, cache = self._caches[run]
             hm = layer.canon(h32, conv_state, dt) if layer.canon is not None else h
             mix = layer.mix(hm, positions, cache)
-            ff = layer.mlp(h) if layer.mlp is not None else None
+            ff = layer.mlp(h, h32) if layer.mlp is not None else None
             nxt = self.layers[self._runs[run + 1]].norm1 if run < last else self.final_norm
             if run == last and logits_rows is not None and streams is None:
                 # only the asked rows go on: the caches and states of this step are complete
