@@ -26,34 +26,61 @@ namespace nv {
 constexpr int kMoeMaxTop = 16;
 constexpr int kMoeBN = 64;
 
+// One wave per token: a lane keeps the logits e = lane, lane + 64, ... in registers (up to kMoeRoutePerLane of them;
+// more experts than that are re-read from memory), and every choice is a wave-wide arg-max (larger value, then lower
+// index) after which the winner's lane strikes its element out.
+constexpr int kMoeRoutePerLane = 8;            // experts <= 512 stay in registers
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int* __restrict__ ids,
                                                         float* __restrict__ wgt, int64_t T, int E, int top) {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= T) return;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;                                // (whole waves leave together)
+    const int lane = threadIdx.x & 63;
     const float* z = logits + t * E;
+    float reg[kMoeRoutePerLane];
+#pragma unroll
+    for (int i = 0; i < kMoeRoutePerLane; ++i) {
+        const int e = lane + 64 * i;
+        reg[i] = e < E ? z[e] : -INFINITY;
+    }
+    unsigned taken = 0;                                // bit i: this lane's element i (of the first 32) is chosen
     int chosen[kMoeMaxTop];
     float val[kMoeMaxTop];
     for (int j = 0; j < top; ++j) {
-        int best = -1;
-        float bv = 0.f;
-        for (int e = 0; e < E; ++e) {
-            bool taken = false;
-            for (int i = 0; i < j; ++i) taken |= chosen[i] == e;
-            const float v = z[e];
-            if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < kMoeRoutePerLane; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && !((taken >> i) & 1u) && (be == 0x7fffffff || reg[i] > bv)) { bv = reg[i]; be = e; }
         }
-        chosen[j] = best;
+        for (int e = lane + 64 * kMoeRoutePerLane; e < E; e += 64) {      // the part that is not in registers
+            bool gone = false;
+            for (int i = 0; i < j; ++i) gone |= chosen[i] == e;
+            const float v = z[e];
+            if (!gone && (be == 0x7fffffff || v > bv)) { bv = v; be = e; }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(bv, off);
+            const int oe = __shfl_xor(be, off);
+            const bool mine_valid = be != 0x7fffffff, other_valid = oe != 0x7fffffff;
+            if (other_valid && (!mine_valid || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
+        }
+        chosen[j] = be;
         val[j] = bv;
+        if ((be & 63) == lane && be < 64 * kMoeRoutePerLane) taken |= 1u << (be >> 6);
     }
-    float sum = 0.f;
-    const float top_logit = val[0];
-    for (int j = 0; j < top; ++j) {
-        val[j] = expf(val[j] - top_logit);
-        sum += val[j];
-    }
-    for (int j = 0; j < top; ++j) {
-        ids[t * top + j] = chosen[j];
-        wgt[t * top + j] = val[j] / sum;
+    if (lane == 0) {
+        float sum = 0.f;
+        const float top_logit = val[0];
+        for (int j = 0; j < top; ++j) {
+            val[j] = expf(val[j] - top_logit);
+            sum += val[j];
+        }
+        for (int j = 0; j < top; ++j) {
+            ids[t * top + j] = chosen[j];
+            wgt[t * top + j] = val[j] / sum;
+        }
     }
 }
 
@@ -244,8 +271,8 @@ extern "C" int nv_moe_route(const float* logits, int32_t* ids, float* weights, i
                "nv_moe_route: top=%d must lie in 1 .. min(E=%d, %d)", top, E, kMoeMaxTop);
     if (T == 0) return NV_OK;
     NV_REQUIRE(logits && ids && weights, NV_ERR_INVALID_ARG, "nv_moe_route: null pointer");
-    NV_REQUIRE((T + 255) / 256 < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_route: launch too large");
-    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, (hipStream_t)stream, logits, ids,
+    NV_REQUIRE((T + 3) / 4 < (1LL << 31), NV_ERR_UNSUPPORTED, "nv_moe_route: launch too large");
+    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((T + 3) / 4)), dim3(256), 0, (hipStream_t)stream, logits, ids,
                        weights, T, E, top);
     return check_launch("nv_moe_route");
 }

@@ -4,7 +4,6 @@ random weights: every kernel of the design next to the like kernel, with its HBM
 throughput of whole models through the engine.  `python bench.py --benarax` prints the record as one JSON line."""
 import argparse
 import json
-import math
 import os
 import sys
 
@@ -31,9 +30,9 @@ def kernel_records(dev):
         rec = {}
         x, a, parts, y = rn(T, W, dtype=torch.float32), rn(T, W), rn(T, 4, W, dtype=torch.float32), rn(T, W)
         w = rn(W, dtype=torch.float32)
-        t = timed(lambda: ops.stream_boundary(x, add=a, add_parts=parts, mult=0.7, copy_dtype=bf))
+        t = timed(lambda: ops.stream_boundary(x, add=a, add_parts=parts, mult=0.5, copy_dtype=bf))
         rec["stream_boundary (mixer + 4 expert parts -> stream, bf16 copy)"] = rate(t, nbytes=T * W * (8 + 2 + 16 + 2))
-        t = timed(lambda: ops.stream_boundary(x, normed=y, normed_weight=w, mult=0.7, norm=w, groups=4, eps=1e-5,
+        t = timed(lambda: ops.stream_boundary(x, normed=y, normed_weight=w, mult=0.5, norm=w, groups=4, eps=1e-5,
                                               out_dtype=bf, want_f32=True))
         rec["stream_boundary (normed side input -> stream -> grouped norm, fp32 + bf16)"] = rate(t, nbytes=T * W * (8 + 2 + 4 + 2))
         h = rn(T, W)
@@ -72,9 +71,8 @@ def kernel_records(dev):
         nv.set_context(None)
         out["recurrent " + name] = rec
 
-    from nanovllm_amd.layers import attention
     Hq = 16
-    for rank, R, Dn in ((96, 32, 64), (192, 64, 128)):
+    for rank, R, Dn in ((128, 32, 96), (192, 64, 128)):
         scale = (Dn + R) ** -0.5
         cases = {"prefill_4x2048": ([2048] * 4, [2048] * 4), "chunk_512_over_8192": ([512], [8192]),
                  "decode_256_seqs_ctx_513_768": ([1] * 256, torch.randint(513, 769, (256,), generator=torch.Generator().manual_seed(1)).tolist()),
@@ -83,7 +81,7 @@ def kernel_records(dev):
             ctx, pos, nb = paged(n_qs, n_ks, bs, dev)
             T = sum(n_qs)
             nv.set_context(ctx)
-            lat = latent_attention.LatentAttention(Hq, rank, R, scale, 1e-5, 1e4, {"factor": 4.0, "fast": 32.0, "slow": 1.0, "original": 4096}, device=dev)
+            lat = latent_attention.LatentAttention(Hq, rank, R, scale, 1e-5, 1e4, {"factor": 8.0, "fast": 16.0, "slow": 2.0, "original": 2048}, device=dev)
             q, q_lat, ckv = rn(T, Hq, Dn + R), rn(T, Hq, rank), rn(T, rank + R)
             kc, vc = rn(nb, bs, 1, rank + R), rn(nb, bs, 1, rank)
             rec = {}
@@ -132,16 +130,16 @@ def kernel_records(dev):
 
 def benarax_config(width, n_groups, vocab, experts=32, top=4, ff=1024):
     mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff, "limit": 7.0}}
-    lat = {"heads": 16, "dim": 64, "rot_dim": 32, "vdim": 64, "q_rank": 768, "kv_rank": 96, "scale": 96 ** -0.5}
+    lat = {"heads": 16, "dim": 96, "rot_dim": 32, "vdim": 96, "q_rank": 768, "kv_rank": 128, "scale": 128 ** -0.5}
     group = [
         {"type": "general_delta", "mlp": mlp, "mixer": {"heads": 16, "dim": 128}},
         {"type": "latent_attention", "mlp": mlp,
-         "mixer": dict(lat, rot={"dims": 32, "base": 1e4, "scaling": {"factor": 4.0, "fast": 32.0, "slow": 1.0, "original": 4096}})},
+         "mixer": dict(lat, rot={"dims": 32, "base": 1e4, "scaling": {"factor": 8.0, "fast": 16.0, "slow": 2.0, "original": 2048}})},
         {"type": "general_delta", "mlp": mlp, "mixer": {"heads": 16, "dim": 128}},
-        {"type": "latent_attention_2", "mlp": mlp, "mixer": dict(lat, rot={"dims": 32, "base": 5e5})},
+        {"type": "latent_attention_2", "mlp": mlp, "mixer": dict(lat, rot={"dims": 32, "base": 1e6})},
     ]
     return {"architecture": "Benarax", "layers": group * n_groups, "norm": {"eps": 1e-5, "groups": 4}, "vocab": vocab,
-            "width": width, "loop": {"start": 0, "stop": 0, "times": 1}, "residual_mult": 0.7, "embedding": {"scale": 1.0},
+            "width": width, "loop": {"start": 0, "stop": 0, "times": 1}, "residual_mult": 0.5, "embedding": {"scale": 1.0},
             "logit_scale": 1.0, "canon": {"taps": 4}, "token_side": {"dim": 64}}
 
 
@@ -169,7 +167,7 @@ def random_benarax(cfg_dict, dev, dtype, rank=64):
 
 def model_records(dev, width=2048, n_groups=2, vocab=32000, batch=32, prompt_len=1024, out_len=64):
     out = {"shape": dict(width=width, layers=4 * n_groups, vocab=vocab, batch=batch, prompt_len=prompt_len, out_len=out_len,
-                         block_size=256, benarax="16 heads; 32 experts, top 4, ff 1024 (active ff 4096); latent 96 + 32",
+                         block_size=256, benarax="16 heads; 32 experts, top 4, ff 1024 (active ff 4096); latent 128 + 32",
                          buvalix="16/8 heads x 128; dense ff 4096")}
     g = torch.Generator().manual_seed(0)
     prompts = [torch.randint(0, vocab, (prompt_len,), generator=g).tolist() for _ in range(batch)]
