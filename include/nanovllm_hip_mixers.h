@@ -74,7 +74,17 @@ NV_API int nv_attn_scoremod_paged(const void* q, const void* k_cache, const void
                                   float softcap, const float* sink, const float* dist_bias, int n_dist,
                                   int max_seqlen_q, int max_seqlen_k, int single_rows, int dtype, int64_t q_stride,
                                   int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream);
-/* Scratch bytes the launch above needs for these sizes (key slices of single rows; 0 when it needs none). */
+/* The same with the value rows `v_row_stride` elements apart (>= Dv; Dv: a dense cache).  A value cache that is a
+ * column range of the key cache (value row = the first Dv columns of the key row, v_row_stride = G * D with G = 1, or
+ * any layout with one stride between consecutive (slot, kv head) rows) is read in place. */
+NV_API int nv_attn_scoremod_paged_vld(const void* q, const void* k_cache, const void* v_cache, int64_t v_row_stride,
+                                      void* out, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                      const int32_t* block_tables, int num_seqs, int max_blocks_per_seq, int64_t T,
+                                      int H, int G, int D, int Dv, int64_t num_blocks, int block_size, float scale,
+                                      float softcap, const float* sink, const float* dist_bias, int n_dist,
+                                      int max_seqlen_q, int max_seqlen_k, int single_rows, int dtype, int64_t q_stride,
+                                      int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream);
+/* Scratch bytes the launches above need for these sizes (key slices of single rows; 0 when it needs none). */
 NV_API int64_t nv_attn_scoremod_workspace_bytes(int num_seqs, int64_t T, int H, int G, int Dv, int max_seqlen_k);
 
 /*
@@ -161,6 +171,7 @@ NV_API int nv_general_delta_rule(const void* r, const void* k, const void* v, in
  * key part shared by all heads (attention in the latent space, G = 1, key size rank + R, value size rank):
  *   c = ckv[t, :rank] / sqrt(mean(.^2) + eps) * latent_w;   k_r = rot(ckv[t, rank:])
  *   q_full[t, h] = [q_lat[t, h] | rot(q[t, h, Dq - R:])];   k_cache[slot] = [c | k_r];   v_cache[slot] = c
+ *   (v_cache NULL: the values are read out of the key rows, nothing else is stored)
  * rot turns pair i by positions[t] * freq[i], cos and sin times mag; pairs (2i, 2i+1) if interleaved else (i, i + R/2).
  * q: [T, H, Dq] (token stride q_stride); q_lat: [T, H, rank] with token / head strides; ckv: [T, rank + R];
  * q_full: [T, H, rank + R] contiguous; k_cache: [num_slots, rank + R]; v_cache: [num_slots, rank].

@@ -73,6 +73,9 @@ MIXERS_PROTOTYPES = {
     "nv_attn_scoremod_paged": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i32, _i32,
                                       _i64, _i32, _f32, _f32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i64, _i64,
                                       _vp, _i64, _vp]),
+    "nv_attn_scoremod_paged_vld": (_i32, [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i64, _i32, _i32, _i32, _i32,
+                                          _i64, _i32, _f32, _f32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i64, _i64,
+                                          _vp, _i64, _vp]),
     "nv_attn_scoremod_workspace_bytes": (_i64, [_i32, _i64, _i32, _i32, _i32, _i32]),
     "nv_causal_conv_silu": (_i32, [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
     "nv_gated_delta_rule": (_i32, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp,

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ cu_k, const int* __restrict__ block_tables, int B,
     int max_blocks, int H, int G, int D, int Dv, int block_size, float scale, float softcap,
     const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride, int only_single_rows) {
+    int64_t out_stride, int64_t v_ld, int only_single_rows) {
     extern __shared__ float smem[];
     float* qs = smem;                      // [D]
     float* ps = smem + D;                  // [64]
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
         for (int i = 0; i < kSmMaxDvPerLane; ++i) acc[i] *= corr;
         for (int jj = 0; jj < n_tile; ++jj) {
             const float pj = ps[jj];
-            const T* vr = v_cache + rows[jj] * Dv;
+            const T* vr = v_cache + rows[jj] * v_ld;
 #pragma unroll
             for (int i = 0; i < kSmMaxDvPerLane; ++i) {
                 const int c = lane + 64 * i;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
     __bf16* __restrict__ out, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int tiles_per_seq, int H, int G, int D, int Dv,
     int block_size, float scale, float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias,
-    int n_dist, int64_t q_stride, int64_t out_stride) {
+    int n_dist, int64_t q_stride, int64_t out_stride, int64_t v_rs) {      // v_rs: elements between value rows
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const int b = blockIdx.x / tiles_per_seq, qt = blockIdx.x % tiles_per_seq, h = blockIdx.y;
     const int q0 = cu_q[b], len_q = cu_q[b + 1] - q0, len_k = cu_k[b + 1] - cu_k[b];
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_scoremod_tile_kernel(
                                                          : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < VP; ++i)
-            vreg[i] = (in && my_quarter + 4 * i < 2 * DVS) ? *(const uint4*)(v_cache + row * Dv + 8 * (my_quarter + 4 * i))
+            vreg[i] = (in && my_quarter + 4 * i < 2 * DVS) ? *(const uint4*)(v_cache + row * v_rs + 8 * (my_quarter + 4 * i))
                                                           : make_uint4(0, 0, 0, 0);
     };
     fetch(0);
@@ -387,7 +387,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
     float* __restrict__ ws, const int* __restrict__ cu_q, const int* __restrict__ cu_k,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int D, int Dv, int block_size, float scale,
     float softcap, const float* __restrict__ sink, const float* __restrict__ dist_bias, int n_dist, int64_t q_stride,
-    int64_t out_stride, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per pass (= REP): sizes the LDS arrays
+    int64_t out_stride, int64_t v_ld, int splits, int slice_keys, int64_t T_rows, int cpr_log2, int repm) {      // repm: heads per pass (= REP): sizes the LDS arrays
     extern __shared__ float dsm[];
     const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
     const int t = cu_q[b];
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(kDecThreads) void attn_scoremod_decode_kernel(
 #pragma unroll 4
                 for (int jj = sub; jj < 64; jj += rows_per_load) {
                     float vv[VN];
-                    load16<T>(v_cache + rw[jj] * Dv + piece * VN, vv);
+                    load16<T>(v_cache + rw[jj] * v_ld + piece * VN, vv);
 #pragma unroll
                     for (int r = 0; r < REP; ++r) {
                         if (r < rep) {
@@ -649,7 +649,7 @@ struct TileArgs {
     float scale, softcap;
     const float *sink, *dist_bias;
     int n_dist;
-    int64_t q_stride, out_stride;
+    int64_t q_stride, out_stride, v_ld;
 };
 template <int DS, int DVS>
 static bool launch_tile_one(dim3 grid, size_t lds, hipStream_t s, const TileArgs& a) {
@@ -664,7 +664,7 @@ static bool launch_tile_one(dim3 grid, size_t lds, hipStream_t s, const TileArgs
     }
     hipLaunchKernelGGL((attn_scoremod_tile_kernel<DS, DVS>), grid, dim3(kTileThreads), lds, s, a.q, a.k_cache, a.v_cache, a.out,
                        a.cu_q, a.cu_k, a.block_tables, a.max_blocks, a.tiles, a.H, a.G, a.D, a.Dv, a.block_size, a.scale,
-                       a.softcap, a.sink, a.dist_bias, a.n_dist, a.q_stride, a.out_stride);
+                       a.softcap, a.sink, a.dist_bias, a.n_dist, a.q_stride, a.out_stride, a.v_ld);
     return true;
 }
 template <int DS>
@@ -693,7 +693,21 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
                                       const float* sink, const float* dist_bias, int n_dist, int max_seqlen_q,
                                       int max_seqlen_k, int single_rows, int dtype, int64_t q_stride,
                                       int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream) {
+    return nv_attn_scoremod_paged_vld(q, k_cache, v_cache, Dv, out, cu_seqlens_q, cu_seqlens_k, block_tables, num_seqs,
+                                      max_blocks_per_seq, T, H, G, D, Dv, num_blocks, block_size, scale, softcap, sink,
+                                      dist_bias, n_dist, max_seqlen_q, max_seqlen_k, single_rows, dtype, q_stride,
+                                      out_stride, workspace, workspace_bytes, stream);
+}
+
+extern "C" int nv_attn_scoremod_paged_vld(const void* q, const void* k_cache, const void* v_cache, int64_t v_ld, void* out,
+                                          const int* cu_seqlens_q, const int* cu_seqlens_k, const int* block_tables,
+                                          int num_seqs, int max_blocks_per_seq, int64_t T, int H, int G, int D, int Dv,
+                                          int64_t num_blocks, int block_size, float scale, float softcap,
+                                          const float* sink, const float* dist_bias, int n_dist, int max_seqlen_q,
+                                          int max_seqlen_k, int single_rows, int dtype, int64_t q_stride,
+                                          int64_t out_stride, void* workspace, int64_t workspace_bytes, void* stream) {
     using namespace nv;
+    NV_REQUIRE(v_ld >= Dv, NV_ERR_INVALID_ARG, "nv_attn_scoremod_paged: value row stride %lld below Dv=%d", (long long)v_ld, Dv);
     NV_REQUIRE(num_seqs >= 0 && T >= 0 && H > 0 && G > 0 && D > 0 && Dv > 0 && block_size > 0 && num_blocks > 0 &&
                    max_blocks_per_seq > 0,
                NV_ERR_INVALID_ARG, "nv_attn_scoremod_paged: bad sizes");
@@ -713,7 +727,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
     // Sequences with several rows: the MFMA tile kernel when the shapes allow (bf16, head sizes in built multiples of
     // 16, aligned rows), else the row-per-wave kernel.
     const size_t tile_lds = sizeof(__bf16) * ((size_t)kTileK * (D + 4) + (size_t)Dv * (kTileK + 4));
-    const bool tile_ok = bf && max_seqlen_q > 1 && tile_built(D) && tile_built(Dv) && D <= 320 && Dv <= 256 &&
+    const bool tile_ok = bf && max_seqlen_q > 1 && tile_built(D) && tile_built(Dv) && D <= 320 && Dv <= 256 && v_ld % 8 == 0 &&
                          tile_lds <= 80 * 1024 && q_stride % 4 == 0 && out_stride % 4 == 0 &&
                          ((uintptr_t)q | (uintptr_t)out) % 8 == 0 && ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
     // Sequences with one row: the decode kernel (key slices, the query heads of a group together) when rows can be
@@ -725,7 +739,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
                            sizeof(int64_t) * 4 * 64;
     int cpr_log2 = 0;                                          // 16-byte pieces per V row, rounded up to a power of two
     while ((vn << cpr_log2) < Dv) ++cpr_log2;
-    const bool dec_ok = singles && D % vn == 0 && Dv % vn == 0 && cpr_log2 <= 6 && dec_lds <= 64 * 1024 &&
+    const bool dec_ok = singles && D % vn == 0 && Dv % vn == 0 && v_ld % vn == 0 && cpr_log2 <= 6 && dec_lds <= 64 * 1024 &&
                         ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
     if (several && tile_ok) {
         const int tiles = (max_seqlen_q + kTileQ - 1) / kTileQ;
@@ -733,7 +747,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
         const dim3 tgrid((unsigned)(num_seqs * tiles), (unsigned)H);
         const TileArgs ta{(const __bf16*)q, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q,
                           cu_seqlens_k, block_tables, max_blocks_per_seq, tiles, H, G, D, Dv, block_size, scale, softcap,
-                          sink, dist_bias, n_dist, q_stride, out_stride};
+                          sink, dist_bias, n_dist, q_stride, out_stride, v_ld};
         NV_REQUIRE(launch_tile(D / 16, Dv / 16, tgrid, tile_lds, s, ta), NV_ERR_LAUNCH,
                    "nv_attn_scoremod_paged: no tile kernel for D=%d, Dv=%d", D, Dv);
         const int rc = check_launch("nv_attn_scoremod_paged (tile kernel)");
@@ -748,7 +762,7 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
 #define NV_DEC_ARGS(TT)                                                                                              \
     (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, (TT*)out, (float*)workspace, cu_seqlens_q, cu_seqlens_k, \
         block_tables, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink, dist_bias, n_dist,        \
-        q_stride, out_stride, plan.splits, plan.slice_keys, T, cpr_log2, repm
+        q_stride, out_stride, v_ld, plan.splits, plan.slice_keys, T, cpr_log2, repm
 #define NV_DEC_LAUNCH(TT, R) \
     hipLaunchKernelGGL((attn_scoremod_decode_kernel<TT, R>), dgrid, dim3(kDecThreads), dec_lds, s, NV_DEC_ARGS(TT))
 #define NV_DEC_BY_REP(TT)                     \
@@ -784,11 +798,11 @@ extern "C" int nv_attn_scoremod_paged(const void* q, const void* k_cache, const 
         hipLaunchKernelGGL(attn_scoremod_rowwave_kernel<__bf16>, grid, dim3(64), smem, s, (const __bf16*)q,
                            (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, cu_seqlens_q, cu_seqlens_k,
                            block_tables, num_seqs, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink,
-                           dist_bias, n_dist, q_stride, out_stride, only);
+                           dist_bias, n_dist, q_stride, out_stride, v_ld, only);
     else
         hipLaunchKernelGGL(attn_scoremod_rowwave_kernel<float>, grid, dim3(64), smem, s, (const float*)q,
                            (const float*)k_cache, (const float*)v_cache, (float*)out, cu_seqlens_q, cu_seqlens_k,
                            block_tables, num_seqs, max_blocks_per_seq, H, G, D, Dv, block_size, scale, softcap, sink,
-                           dist_bias, n_dist, q_stride, out_stride, only);
+                           dist_bias, n_dist, q_stride, out_stride, v_ld, only);
     return check_launch("nv_attn_scoremod_paged");
 }

@@ -9,7 +9,8 @@
 //     c        = ckv[t, :rank] / sqrt(mean(ckv[t, :rank]^2) + eps) * latent_w          (fp32, then the cache dtype)
 //     k_r      = rot_p(ckv[t, rank:])
 //     q_full[t, h] = [q_lat[t, h] | rot_p(q[t, h, Dq - R:])]
-//     k_cache[slot(t)] = [c | k_r],   v_cache[slot(t)] = c                             (slot < 0: not stored)
+//     k_cache[slot(t)] = [c | k_r],   v_cache[slot(t)] = c                             (slot < 0: not stored; v_cache
+//                                                                                       absent: values alias the keys)
 // rot_p turns pair i by the angle p * freq[i] (fp32 product) with cos and sin both times `mag`; the pair is
 // (2i, 2i+1) when `interleaved`, else (i, i + R/2).  The frequencies are a table of the caller's (plain powers of a
 // base, or blended for long contexts).
@@ -48,11 +49,10 @@ __global__ __launch_bounds__(256) void latent_prep_store_kernel(
     const int64_t slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
     if (slot >= 0) {
         T* krow = k_cache + slot * Dk;
-        T* vrow = v_cache + slot * rank;
         for (int c = tid; c < rank; c += 256) {
             const T v = (T)((float)crow[c] * rstd * latent_w[c]);
             krow[c] = v;
-            vrow[c] = v;
+            if (v_cache != nullptr) v_cache[slot * rank + c] = v;      // (absent when the values alias the key rows)
         }
         for (int i = tid; i < half; i += 256) {
             const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
@@ -87,7 +87,7 @@ extern "C" int nv_latent_prep_store(const void* q, int64_t q_stride, int Dq, con
     if (T == 0) return NV_OK;
     NV_REQUIRE(q && q_lat && ckv && latent_w && positions && q_full, NV_ERR_INVALID_ARG,
                "nv_latent_prep_store: null pointer");
-    NV_REQUIRE(!slot_mapping || (k_cache && v_cache), NV_ERR_INVALID_ARG, "nv_latent_prep_store: scatter needs the caches");
+    NV_REQUIRE(!slot_mapping || k_cache, NV_ERR_INVALID_ARG, "nv_latent_prep_store: scatter needs the key cache");
     NV_REQUIRE(R % 2 == 0 && R <= 1024 && (R == 0 || freq), NV_ERR_INVALID_ARG,
                "nv_latent_prep_store: the rotated part (%d) must be even, at most 1024, with its frequencies", R);
     NV_REQUIRE(dtype == NV_DTYPE_BF16 || dtype == NV_DTYPE_F32, NV_ERR_INVALID_ARG, "nv_latent_prep_store: bad dtype");

@@ -262,7 +262,11 @@ class ModelRunner:
         for spec in self.cache_specs:
             if isinstance(spec, PagedKVSpec):
                 k = torch.zeros(num_blocks, self.block_size, spec.kv_heads, spec.key_dim, dtype=self.dtype, device=self.device)
-                v = torch.zeros(num_blocks, self.block_size, spec.kv_heads, spec.value_dim, dtype=self.dtype, device=self.device)
+                if spec.value_in_key:
+                    v = k[..., :spec.value_dim]
+                else:
+                    v = torch.zeros(num_blocks, self.block_size, spec.kv_heads, spec.value_dim, dtype=self.dtype,
+                                    device=self.device)
                 caches.append((k, v))
             else:
                 caches.append({name: torch.zeros((self.num_state_slots,) + tuple(shape), dtype=dt or self.dtype,

@@ -55,7 +55,8 @@ class LatentAttention(nn.Module):
     def forward(self, q: torch.Tensor, q_lat: torch.Tensor, ckv: torch.Tensor, positions: torch.Tensor,
                 k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
         """q [T, H, Dq] (its last R columns get the rotary); q_lat [T, H, rank]; ckv [T, rank + R] as projected;
-        k_cache [num_blocks, block_size, 1, rank + R], v_cache [.., 1, rank].  Returns [T, H, rank]."""
+        k_cache [num_blocks, block_size, 1, rank + R]; v_cache [.., 1, rank]: a cache of its own, or the first `rank`
+        columns of k_cache (then nothing is stored twice).  Returns [T, H, rank]."""
         ctx = get_context()
         q_full = ops.latent_prep_store(q, q_lat, ckv, self.latent_norm, self.freq, self.mag, self.interleaved, positions,
                                        ctx.slot_mapping, k_cache, v_cache, self.rot_dim, self.eps)

@@ -200,8 +200,8 @@ class BenaraxLatentAttention(nn.Module, _FusedInputs):
                                       interleaved=LATENT_KINDS[m.kind], device=device)
 
     def cache_spec(self):
-        # one key "head" [latent | rotated part] and the latent again as its value
-        return PagedKVSpec(1, self.m.kv_rank + self.m.rot_dim, self.m.kv_rank)
+        # one key "head" [latent | rotated part]; the value of a token is the latent, i.e. the front of its key row
+        return PagedKVSpec(1, self.m.kv_rank + self.m.rot_dim, self.m.kv_rank, value_in_key=True)
 
     def finalize(self):
         self._fuse(self._inputs)

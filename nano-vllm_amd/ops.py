@@ -472,11 +472,16 @@ def attn_scoremod_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     dt = _dt(q, "q")
     _rows_ok(q, "q")
     T, H, D = q.shape
-    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.is_contiguous() and v_cache.is_contiguous()
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.is_contiguous()
           and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[:3] == v_cache.shape[:3]
-          and k_cache.shape[3] == D, "caches must be contiguous [num_blocks, block_size, G, D | Dv] of q's dtype")
+          and k_cache.shape[3] == D, "caches must be [num_blocks, block_size, G, D | Dv] of q's dtype, the keys contiguous")
     nb, bs, G, _ = k_cache.shape
     Dv = v_cache.shape[3]
+    # value rows: dense, or any layout with ONE stride between consecutive (slot, kv head) rows, e.g. a column range of
+    # the key cache
+    v_ld = v_cache.stride(2)
+    _need(v_cache.stride(3) == 1 and v_ld >= Dv and v_cache.stride(1) == G * v_ld and v_cache.stride(0) == bs * G * v_ld,
+          "value rows must be evenly spaced (a dense cache or a column range of one)")
     _i32(cu_seqlens_q, "cu_seqlens_q")
     _i32(cu_seqlens_k, "cu_seqlens_k")
     B = cu_seqlens_k.numel() - 1
@@ -494,7 +499,7 @@ def attn_scoremod_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     dll = _lib.mixers()
     need = dll.nv_attn_scoremod_workspace_bytes(B, T, H, G, Dv, int(max_seqlen_k))
     ws = _workspace(q.device, need) if need else None
-    rc = dll.nv_attn_scoremod_paged(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+    rc = dll.nv_attn_scoremod_paged_vld(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), v_ld, out.data_ptr(),
                                     cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), block_tables.data_ptr(), B,
                                     block_tables.shape[1], T, H, G, D, Dv, nb, bs, float(scale), float(softcap or 0.0),
                                     _f32c(sink, "sink") or None, _f32c(dist_bias, "dist_bias") or None, n_dist,
@@ -727,16 +732,22 @@ def latent_prep_store(q: torch.Tensor, q_lat: torch.Tensor, ckv: torch.Tensor, l
     if slot_mapping is not None:
         _i32(slot_mapping, "slot_mapping")
         _need(slot_mapping.numel() == T, "slot_mapping length != number of tokens")
-        _need(k_cache is not None and v_cache is not None and k_cache.is_contiguous() and v_cache.is_contiguous()
-              and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.shape[2:] == (1, rank + R)
-              and v_cache.shape[2:] == (1, rank) and k_cache.shape[:2] == v_cache.shape[:2],
-              "caches must be contiguous [num_blocks, block_size, 1, rank + R] and [.., 1, rank] of q's dtype")
+        _need(k_cache is not None and k_cache.is_contiguous() and k_cache.dtype == q.dtype
+              and k_cache.shape[2:] == (1, rank + R), "k_cache must be contiguous [num_blocks, block_size, 1, rank + R] of q's dtype")
+        if v_cache is not None and v_cache.data_ptr() == k_cache.data_ptr():
+            _need(v_cache.shape == k_cache.shape[:3] + (rank,) and v_cache.stride() == k_cache.stride(),
+                  "a value cache inside the key cache must be its first `rank` columns")
+            v_cache = None                    # the values are the front of the key rows: nothing else to store
+        else:
+            _need(v_cache is not None and v_cache.is_contiguous() and v_cache.dtype == q.dtype
+                  and v_cache.shape == k_cache.shape[:3] + (rank,), "v_cache must be contiguous [.., 1, rank] of q's dtype")
     q_full = torch.empty((T, H, rank + R), dtype=q.dtype, device=q.device)
     dll = _lib.mixers()
     rc = dll.nv_latent_prep_store(q.data_ptr(), q.stride(0), Dq, q_lat.data_ptr(), q_lat.stride(0), q_lat.stride(1),
                                   ckv.data_ptr(), ckv.stride(0), _f32c(latent_weight, "latent_weight"),
                                   _f32c(freq, "freq") or None, float(mag), int(bool(interleaved)), positions.data_ptr(),
-                                  _ptr(slot_mapping), q_full.data_ptr(), _ptr(k_cache), _ptr(v_cache), dt, T, H, rank, R,
+                                  _ptr(slot_mapping), q_full.data_ptr(), _ptr(k_cache),
+                                  _ptr(v_cache) if slot_mapping is not None else None, dt, T, H, rank, R,
                                   float(eps), _stream(q))
     _lib.check(rc, "nv_latent_prep_store", dll)
     return q_full

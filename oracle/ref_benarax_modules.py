@@ -163,7 +163,8 @@ class LatentAttention(nn.Module):
         bs = k_cache.shape[1]
         slots = ctx.slot_mapping.long()
         k_cache.view(-1, rank + R)[slots] = torch.cat([c, k_rot], dim=-1)
-        v_cache.view(-1, rank)[slots] = c
+        if v_cache.data_ptr() != k_cache.data_ptr():      # (else the values are the front of the key rows)
+            v_cache.view(-1, rank)[slots] = c
         cu_q, cu_k = ctx.cu_seqlens_q.tolist(), ctx.cu_seqlens_k.tolist()
         out = torch.zeros(T, H, rank, dtype=torch.float32, device=q.device)
         for b in range(len(cu_q) - 1):
@@ -172,7 +173,7 @@ class LatentAttention(nn.Module):
                 continue
             pos_k = torch.arange(nk, device=q.device)
             rows = ctx.block_tables[b].long()[pos_k // bs] * bs + pos_k % bs
-            kk, vv = k_cache.view(-1, rank + R)[rows].float(), v_cache.view(-1, rank)[rows].float()
+            kk, vv = k_cache.view(-1, rank + R)[rows].float(), v_cache.reshape(-1, rank)[rows].float()
             pos_q = nk - nq + torch.arange(nq, device=q.device)
             s = torch.einsum("ihd,jd->hij", q_full[cu_q[b]:cu_q[b + 1]].float(), kk) * self.scale
             s = s.masked_fill((pos_q[:, None] < pos_k[None, :])[None], float("-inf"))

@@ -194,7 +194,7 @@ def test_far_key_own_position_and_next_position(dev, interleaved):
     for cuts in cuts_for(T) + [[148, 1, 1, 1, 1, 148]]:
         nb = -(-T // 8) + 2
         kc = torch.full((nb, 8, 1, rank + Rr), 9.0, device=dev)
-        vc = torch.full((nb, 8, 1, rank), -9.0, device=dev)
+        vc = kc[..., :rank]                          # the values are the front of the key rows, as in the engine
         got = in_portions(dev, lambda s, p: attn(q[s].to(dev), q_lat[s].to(dev), ckv[s].to(dev), p, kc, vc), T, cuts)
         torch.testing.assert_close(got, want, rtol=2e-4, atol=2e-4)
 

@@ -103,7 +103,8 @@ def test_general_delta_rule(dt, step, H, D):
     (4, 80, 16, 48, True, {"factor": 3.0, "fast": 16.0, "slow": 2.0, "original": 128}),     # key 96, value 80: tile kernel
     (3, 40, 8, 24, False, None),                                                            # single rows by 16-byte pieces
     (2, 64, 64, 32, False, None), (5, 18, 6, 10, True, None), (2, 192, 64, 128, True, None)])
-def test_latent_attention(dt, step, H, rank, Rr, Dn, inter, scaling):
+@pytest.mark.parametrize("alias", [False, True], ids=["own-values", "values-in-keys"])
+def test_latent_attention(dt, step, H, rank, Rr, Dn, inter, scaling, alias):
     L, g, (T, pos) = hip_layers(), torch.Generator().manual_seed(rank), step
     la = L.LatentAttention(H, rank, Rr, 0.1, 1e-5, 5000.0, scaling, interleaved=inter, device=DEV)
     lb = R.LatentAttention(H, rank, Rr, 0.1, 1e-5, 5000.0, scaling, interleaved=inter, device=DEV)
@@ -112,8 +113,8 @@ def test_latent_attention(dt, step, H, rank, Rr, Dn, inter, scaling):
     lb.latent_norm.data.copy_(v)
     q, ql, ckv = rn(g, T, H, Dn + Rr).to(dt), rn(g, H, T, rank).to(dt).transpose(0, 1), rn(g, T, rank + Rr).to(dt)
     ka = rn(g, 40, 8, 1, rank + Rr).to(dt)
-    va = ka[..., :rank].contiguous().clone()
-    kb, vb = ka.clone(), va.clone()
+    kb = ka.clone()
+    va, vb = (ka[..., :rank], kb[..., :rank]) if alias else (ka[..., :rank].contiguous().clone(), ka[..., :rank].contiguous().clone())
     oa, ob = la(q, ql, ckv, pos, ka, va), lb(q, ql, ckv, pos, kb, vb)
     assert rel(oa, ob) < (1e-5 if dt == torch.float32 else 2e-2)
     assert rel(ka, kb) < tol(dt) and rel(va, vb) < tol(dt)

@@ -83,15 +83,16 @@ def kernel_records(dev):
             nv.set_context(ctx)
             lat = latent_attention.LatentAttention(Hq, rank, R, scale, 1e-5, 1e4, {"factor": 8.0, "fast": 16.0, "slow": 2.0, "original": 2048}, device=dev)
             q, q_lat, ckv = rn(T, Hq, Dn + R), rn(T, Hq, rank), rn(T, rank + R)
-            kc, vc = rn(nb, bs, 1, rank + R), rn(nb, bs, 1, rank)
+            kc = rn(nb, bs, 1, rank + R)
+            vc = kc[..., :rank]                      # the values are the front of the key rows
             rec = {}
             t = timed(lambda: ops.latent_prep_store(q, q_lat, ckv, lat.latent_norm, lat.freq, lat.mag, True, pos,
                                                     ctx.slot_mapping, kc, vc, R, 1e-5))
-            rec["latent_prep_store"] = rate(t, nbytes=T * (Hq * (rank + R) * 4 + (rank + R) * 2 * 3))
+            rec["latent_prep_store"] = rate(t, nbytes=T * (Hq * (rank + R) * 4 + (rank + R) * 2 * 2))
             qf = rn(T, Hq, rank + R)
             pairs = sum(nq * (nk - nq) + nq * (nq + 1) // 2 for nq, nk in zip(n_qs, n_ks))
             flops = 2 * (rank + R + rank) * Hq * pairs
-            kv_bytes = sum(n_ks) * (2 * rank + R) * 2 + T * Hq * (2 * rank + R) * 2
+            kv_bytes = sum(n_ks) * (rank + R) * 2 + T * Hq * (2 * rank + R) * 2
             singles = int(max(n_qs) == 1)
             t = timed(lambda: ops.attn_scoremod_paged(qf, kc, vc, ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.block_tables, scale,
                                                       0.0, None, None, max(n_qs), max(n_ks), singles), iters=5)
