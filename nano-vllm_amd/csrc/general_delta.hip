@@ -12,7 +12,8 @@
 // (sequence, head); a lane owns one value column and a quarter of the key rows (its quad index r owns rows
 // r * RPL .. r * RPL + RPL - 1, read from LDS four at a time, the four runs RPL + 4 words apart so that a quad's 16-byte
 // reads fall on different banks), so the state lives in registers and the token loop has no workgroup barrier: the
-// vectors of up to 16 tokens are prepared into LDS by all waves together, each wave then runs those tokens for its 16
+// vectors of up to 16 tokens are prepared into LDS by all waves together (every load of the tile issued at once, then the
+// unit keys per token), each wave then runs those tokens for its 16
 // columns (one pass for u^T S, one for the update and the read-out, a two-step quad reduction each), and the
 // normalised, gated read-out of the tile is written by all waves together.
 #include <algorithm>
@@ -66,35 +67,42 @@ __global__ void general_delta_rule_kernel(
     for (int t0 = 0; t0 < len_q; t0 += tile) {
         const int nt = min(tile, len_q - t0);
         __syncthreads();                              // the previous tile's epilogue has read os
-        // ---- prepare the tile ------------------------------------------------------------------------------
+        // ---- prepare the tile: all loads of the tile in flight at once, then the unit keys per token -------
+        for (int i = tid; i < nt * 4 * RPL; i += blockDim.x) {
+            const int tt = i / (4 * RPL), d = i % (4 * RPL);
+            const int at = tt * DP + (d / RPL) * (RPL + 4) + (d % RPL);
+            float wv = 1.f, av = 0.f, kv = 0.f, rv = 0.f;
+            if (d < D) {
+                const int64_t t = q0 + t0 + tt, hd = (int64_t)h * D + d;
+                kv = (float)k[t * k_stride + hd];
+                rv = (float)r_in[t * r_stride + hd];
+                wv = expf(-decay_rate * gd_sigmoid((float)w_raw[t * w_stride + hd] + w_bias[hd]));
+                av = gd_sigmoid((float)a_raw[t * a_stride + hd] + a_bias[hd]);
+            }
+            ws[at] = wv;
+            as[at] = av;
+            ks[at] = kv;
+            rs[at] = rv;
+        }
+        for (int i = tid; i < nt * D; i += blockDim.x) {
+            const int tt = i / D, c = i % D;
+            vs[tt * D + c] = (float)v[(int64_t)(q0 + t0 + tt) * v_stride + (int64_t)h * D + c];
+        }
+        __syncthreads();
         for (int tt = wave; tt < nt; tt += n_waves) {
-            const int64_t t = q0 + t0 + tt;
-            const T* kr = k + t * k_stride + (int64_t)h * D;
             float kk = 0.f;
-            for (int d = lane; d < D; d += 64) {
-                const float kv = (float)kr[d];
+            for (int d = lane; d < 4 * RPL; d += 64) {
+                const float kv = ks[tt * DP + (d / RPL) * (RPL + 4) + (d % RPL)];     // (zeros past D)
                 kk += kv * kv;
             }
             kk = wave_sum(kk);
             const float kn = 1.0f / sqrtf(kk + key_eps);
             for (int d = lane; d < 4 * RPL; d += 64) {
                 const int at = tt * DP + (d / RPL) * (RPL + 4) + (d % RPL);
-                float uv = 0.f, wv = 1.f, av = 0.f, kv = 0.f, rv = 0.f;
-                if (d < D) {
-                    const int64_t hd = (int64_t)h * D + d;
-                    kv = (float)kr[d];
-                    uv = kv * kn;
-                    rv = (float)r_in[t * r_stride + hd];
-                    wv = expf(-decay_rate * gd_sigmoid((float)w_raw[t * w_stride + hd] + w_bias[hd]));
-                    av = gd_sigmoid((float)a_raw[t * a_stride + hd] + a_bias[hd]) * uv;
-                }
+                const float uv = ks[at] * kn;
                 us[at] = uv;
-                ws[at] = wv;
-                as[at] = av;
-                ks[at] = kv;
-                rs[at] = rv;
+                as[at] *= uv;
             }
-            for (int c = lane; c < D; c += 64) vs[tt * D + c] = (float)v[t * v_stride + (int64_t)h * D + c];
         }
         __syncthreads();
         // ---- the recurrence over the tile, no barrier inside ---------------------------------------------

@@ -130,3 +130,26 @@ def test_routed_experts(dt, E, top, ff, T, W):
     oa, ob = L.MoEExperts(top, 0.8)(h, lg, gu, dn), R.MoEExperts(top, 0.8)(h, lg, gu, dn)
     assert oa.shape == (T, top, W) and oa.dtype == torch.float32
     assert rel(oa, ob) < (1e-5 if dt == torch.float32 else 1e-2)
+
+
+def test_general_delta_rule_many_pairs(dt):
+    """Enough (sequence, head) pairs that every head stays in one workgroup (fewer pairs split a head's columns)."""
+    L, g = hip_layers(), torch.Generator().manual_seed(3)
+    B, H, D = 140, 4, 32
+    n_q = [1] * (B - 2) + [3, 2]
+    n_k = [q + (i % 5) for i, q in enumerate(n_q)]
+    ctx, _ = paged_context(n_q, n_k, 8, 2 * B, 2, DEV, slots=list(range(B))[::-1])
+    nv.set_context(ctx)
+    T = sum(n_q)
+    da, db = L.GeneralDeltaRule(H, D, 1e-5, device=DEV), R.GeneralDeltaRule(H, D, 1e-5, device=DEV)
+    for n in ("a_bias", "w_bias", "norm_weight"):
+        v = rn(g, H * D)
+        getattr(da, n).data.copy_(v)
+        getattr(db, n).data.copy_(v)
+    r, k, v = (rn(g, T, H, D).to(dt) for _ in range(3))
+    w_raw, a_raw, gate = (rn(g, T, H * D).to(dt) for _ in range(3))
+    sa = rn(g, B, H, D, D) * 0.3
+    sb = sa.clone()
+    assert rel(da(r, k, v, w_raw, a_raw, gate, sa), db(r, k, v, w_raw, a_raw, gate, sb)) < max(tol(dt), 2e-5)
+    assert rel(sa, sb) < 1e-5
+    nv.set_context(None)
