@@ -60,7 +60,7 @@ NV_API int nv_qk_prep_store(const void* q, const void* k, const void* v, void* q
  *   dist_bias;  the softmax denominator also holds exp(sink[h]) if sink.
  * q: [T, H, D] (token stride q_stride), out: [T, H, Dv] (token stride out_stride);
  * k_cache: [num_blocks, block_size, G, D], v_cache: [num_blocks, block_size, G, Dv]; query i of sequence b sits at
- * position len_k(b) - len_q(b) + i.  Dv <= 256.
+ * position len_k(b) - len_q(b) + i.  Dv <= 512 (above 256 on the row-per-wave kernel only).
  * max_seqlen_q / max_seqlen_k: the most rows / keys any sequence has in this step (0 = unknown).  Three kernels
  * share the work: sequences with several rows run on a bf16 MFMA tile kernel (head sizes: multiples of 16 up to 128, of 32 up to 320 / 256) sized from
  * max_seqlen_q; sequences with one row on a decode kernel that reads K/V once per group of query heads and cuts long

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void qk_prep_store_kernel(
 // One wave per (query token, query head).  Keys go by in tiles of 64: lane j scores key j of the tile (its own
 // K row, q broadcast from LDS), the tile's weights go through LDS, then the lanes switch to value channels
 // (lane c accumulates channels c, c + 64, ...) and stream the tile's V rows, which are contiguous per key.
-constexpr int kSmMaxDvPerLane = 4;   // Dv <= 256
+constexpr int kSmMaxDvPerLane = 8;   // Dv <= 512 (the tile and decode kernels take Dv <= 256, the row-per-wave kernel the rest)
 
 template <typename T>
 __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(64) void attn_scoremod_rowwave_kernel(
     const int* table = block_tables + (int64_t)b * max_blocks;
     const float* bias_h = dist_bias ? dist_bias + (int64_t)h * n_dist : nullptr;
     float m = -INFINITY, l = 0.f;
-    float acc[kSmMaxDvPerLane] = {0.f, 0.f, 0.f, 0.f};
+    float acc[kSmMaxDvPerLane] = {};
     const int n_keys = pos + 1;
     __syncthreads();
     for (int base = 0; base < n_keys; base += 64) {
@@ -739,7 +739,7 @@ extern "C" int nv_attn_scoremod_paged_vld(const void* q, const void* k_cache, co
                            sizeof(int64_t) * 4 * 64;
     int cpr_log2 = 0;                                          // 16-byte pieces per V row, rounded up to a power of two
     while ((vn << cpr_log2) < Dv) ++cpr_log2;
-    const bool dec_ok = singles && D % vn == 0 && Dv % vn == 0 && v_ld % vn == 0 && cpr_log2 <= 6 && dec_lds <= 64 * 1024 &&
+    const bool dec_ok = singles && D % vn == 0 && Dv % vn == 0 && Dv <= 256 && v_ld % vn == 0 && cpr_log2 <= 6 && dec_lds <= 64 * 1024 &&
                         ((uintptr_t)k_cache | (uintptr_t)v_cache) % 16 == 0;
     if (several && tile_ok) {
         const int tiles = (max_seqlen_q + kTileQ - 1) / kTileQ;
