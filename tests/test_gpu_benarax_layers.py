@@ -103,7 +103,8 @@ def test_general_delta_rule(dt, step, H, D):
     (4, 80, 16, 48, True, {"factor": 3.0, "fast": 16.0, "slow": 2.0, "original": 128}),     # key 96, value 80: tile kernel
     (3, 40, 8, 24, False, None),                                                            # single rows by 16-byte pieces
     (2, 64, 64, 32, False, None), (5, 18, 6, 10, True, None), (2, 192, 64, 128, True, None),
-    (2, 320, 16, 40, False, None)])                                                          # values wider than 256
+    (2, 320, 16, 40, False, None),                                                          # values wider than 256
+    (2, 256, 64, 32, True, None)])                                                           # the largest tile shape (320 / 256)
 @pytest.mark.parametrize("alias", [False, True], ids=["own-values", "values-in-keys"])
 def test_latent_attention(dt, step, H, rank, Rr, Dn, inter, scaling, alias):
     L, g, (T, pos) = hip_layers(), torch.Generator().manual_seed(rank), step
