@@ -122,7 +122,7 @@ def test_latent_attention(dt, step, H, rank, Rr, Dn, inter, scaling, alias):
     assert rel(ka, kb) < tol(dt) and rel(va, vb) < tol(dt)
 
 
-@pytest.mark.parametrize("E,top,ff,T,W", [(16, 2, 64, 25, 96), (5, 3, 24, 25, 100), (8, 2, 40, 700, 96), (4, 4, 16, 3, 36),
+@pytest.mark.parametrize("E,top,ff,T,W", [(14, 2, 56, 25, 96), (5, 3, 24, 25, 100), (8, 2, 40, 700, 96), (4, 4, 16, 3, 36),
                                           (12, 1, 72, 130, 256), (6, 2, 200, 2000, 128), (600, 3, 8, 40, 64), (70, 16, 8, 9, 32)])
 def test_routed_experts(dt, E, top, ff, T, W):
     L, g = hip_layers(), torch.Generator().manual_seed(E)
